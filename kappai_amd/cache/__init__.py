@@ -1,7 +1,7 @@
-from .manager import (CacheError, CacheManager, OutOfPages, OutOfSlots, PageAllocator,
+from .manager import (BundleView, CacheError, CacheManager, OutOfPages, OutOfSlots, PageAllocator,
                       PagedLayerView, RequestCache, StateLayerView)
-from .specs import FixedState, PagedKV, PagedSpec, PoolSpec
+from .specs import CacheBundle, FixedState, PagedKV, PagedSpec, PoolSpec
 
-__all__ = ["CacheError", "CacheManager", "OutOfPages", "OutOfSlots", "PageAllocator",
+__all__ = ["BundleView", "CacheBundle", "CacheError", "CacheManager", "OutOfPages", "OutOfSlots", "PageAllocator",
            "PagedLayerView", "RequestCache", "StateLayerView", "FixedState", "PagedKV",
            "PagedSpec", "PoolSpec"]

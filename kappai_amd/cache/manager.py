@@ -20,7 +20,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Union
 import numpy as np
 import torch
 
-from .specs import FixedState, PagedSpec
+from .specs import CacheBundle, FixedState, PagedSpec
 
 
 class CacheError(RuntimeError):
@@ -125,6 +125,16 @@ class StateLayerView:
     spec: FixedState
 
 
+@dataclass
+class BundleView:
+    """What a layer sees that asked for a ``CacheBundle``: its members' views by their names
+    (None for a member that asked for nothing)."""
+    parts: Dict[str, object]
+
+    def part(self, name: str):
+        return self.parts[name]
+
+
 class RequestCache:
     """Everything one live request holds: a slot, and per paged group its block table.
     ``length`` counts the tokens whose keys are stored."""
@@ -152,7 +162,7 @@ class RequestCache:
         return f"RequestCache({self.request_id!r}, slot={self.slot}, length={self.length})"
 
 
-Spec = Union[PagedSpec, FixedState, None]
+Spec = Union[PagedSpec, FixedState, CacheBundle, None]
 
 
 class CacheManager:
@@ -169,8 +179,15 @@ class CacheManager:
         self.cache_specs = list(cache_specs)
         self.paged_groups: List[PagedGroup] = []
         self.state_groups: List[StateGroup] = []
-        self._where: Dict[int, tuple] = {}
+        self._where: Dict[Hashable, tuple] = {}
+        # a bundle's members are caches of their own under the key (cache id, member's name)
+        asked = []
         for cid, spec in enumerate(self.cache_specs):
+            if isinstance(spec, CacheBundle):
+                asked += [((cid, name), member) for name, member in spec.parts]
+            else:
+                asked.append((cid, spec))
+        for cid, spec in asked:
             if spec is None:
                 continue
             if isinstance(spec, PagedSpec):
@@ -241,7 +258,10 @@ class CacheManager:
         return sum(g.spec.bytes_per_token(dtype_bytes) * len(g.cache_ids)
                    for g in self.paged_groups)
 
-    def view(self, cache_id: int):
+    def view(self, cache_id):
+        if isinstance(cache_id, int) and isinstance(self.cache_specs[cache_id], CacheBundle):
+            return BundleView({name: (None if member is None else self.view((cache_id, name)))
+                               for name, member in self.cache_specs[cache_id].parts})
         if cache_id not in self._where:
             raise CacheError(f"cache {cache_id} was declared to need nothing")
         kind, gi = self._where[cache_id]
@@ -252,7 +272,7 @@ class CacheManager:
         return StateLayerView(g.states.get(cache_id), gi, g.spec)
 
     # -- looking into a request's cache ------------------------------------------------------
-    def export_range(self, rc: RequestCache, cache_id: int, pos_start: int = 0,
+    def export_range(self, rc: RequestCache, cache_id, pos_start: int = 0,
                      n_rows: Optional[int] = None) -> Dict[str, torch.Tensor]:
         """What the paged cache ``cache_id`` holds for positions ``pos_start .. pos_start +
         n_rows - 1`` of the request, gathered out of its pages: ``{pool name: [n_rows, *rest]}``
@@ -286,7 +306,7 @@ class CacheManager:
             out[pool.name] = moved[pages.to(t.device), slots.to(t.device)].clone()
         return out
 
-    def export_state(self, rc: RequestCache, cache_id: int) -> torch.Tensor:
+    def export_state(self, rc: RequestCache, cache_id) -> torch.Tensor:
         """A copy of the request's slot of the fixed-size state ``cache_id`` (kappai:
         kvcache_export_state, src/kvcache.c:924-945)."""
         self._check_live(rc)
@@ -304,7 +324,8 @@ class CacheManager:
         self._check_live(rc)
         out = {"request": rc.request_id, "length": rc.length, "slot": rc.slot,
                "blocks": [list(b) for b in rc.blocks], "caches": {}}
-        for cid, (kind, gi) in sorted(self._where.items()):
+        for cid, (kind, gi) in sorted(self._where.items(), key=lambda kv: (
+                (kv[0], "") if isinstance(kv[0], int) else kv[0])):
             if kind == "state":
                 out["caches"][cid] = {"kind": "state", "state": self.export_state(rc, cid)}
                 continue

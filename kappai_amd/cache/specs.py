@@ -66,3 +66,19 @@ class FixedState:
     so slots are not cleared between requests (src/recipe/ops_hybrid.c:353-354)."""
     shape: Tuple[int, ...]
     dtype: str = "float32"
+
+
+@dataclass(frozen=True)
+class CacheBundle:
+    """Several needs of one layer, each under a name of the layer's choosing: a mixer's keys and
+    values beside the short histories of the convolutions in front of its sublayers, say.  The
+    manager serves every member as if a layer of its own had asked for it; the layer's view is a
+    ``BundleView`` whose ``part(name)`` is the member's view.  ``window`` is that of the paged
+    members (they share the request's block tables only with their equals, as always)."""
+    parts: Tuple[Tuple[str, object], ...]
+
+    def member(self, name: str):
+        for n, spec in self.parts:
+            if n == name:
+                return spec
+        raise KeyError(name)

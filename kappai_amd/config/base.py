@@ -154,6 +154,10 @@ def lookup_architecture(name: str) -> Architecture:
 
 
 def architecture_name(raw: Dict[str, Any]) -> str:
+    """``architectures[0]``, or the single name under ``architecture``."""
+    single = raw.get("architecture")
+    if "architectures" not in raw and isinstance(single, str) and single:
+        return single
     archs = raw.get("architectures")
     if not isinstance(archs, list) or not archs or not isinstance(archs[0], str):
         raise ConfigError("config.json: key 'architectures' must be a list that starts with the "

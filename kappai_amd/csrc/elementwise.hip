@@ -383,6 +383,41 @@ extern "C" int kappai_swiglu(const void* gu, void* act, int T, int F, int is_bf1
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
+// act(gate) * up with a choice of act: 0 silu, 1 the tanh form of gelu,
+// 0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))).
+template <typename T>
+__global__ void glu_kernel(const T* __restrict__ gu, T* __restrict__ act, int F, size_t n,
+                           int kind) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const size_t t = i / F;
+  const int f = (int)(i - t * F);
+  const float g = to_f32(gu[t * 2 * F + f]);
+  const float u = to_f32(gu[t * 2 * F + F + f]);
+  float a;
+  if (kind == 1)
+    a = 0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g)));
+  else
+    a = g / (1.0f + expf(-g));
+  from_f32(act + i, a * u);
+}
+
+extern "C" int kappai_glu(const void* gu, void* act, int T, int F, int is_bf16, int kind,
+                          hipStream_t stream) {
+  const size_t n = (size_t)T * F;
+  if (n == 0) return 0;
+  if (kind < 0 || kind > 1) return (int)hipErrorInvalidValue;
+  const int threads = 256;
+  const unsigned blocks = (unsigned)((n + threads - 1) / threads);
+  if (is_bf16)
+    hipLaunchKernelGGL(glu_kernel<bf16_t>, dim3(blocks), dim3(threads), 0, stream,
+                       (const bf16_t*)gu, (bf16_t*)act, F, n, kind);
+  else
+    hipLaunchKernelGGL(glu_kernel<float>, dim3(blocks), dim3(threads), 0, stream,
+                       (const float*)gu, (float*)act, F, n, kind);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
 // ---------------------------------------------------------------------------------------
 // casts between float and bf16 (activations that meet a matrix stored in 32 bits)
 // ---------------------------------------------------------------------------------------

@@ -125,8 +125,19 @@ __device__ __forceinline__ void store_out(bf16_t* p, float v) { *p = f32_to_bf16
 // (each good to about an ulp of float, far below a bfloat16's rounding) instead of expf and a
 // division, which were 9 of the 132 us of gate/up at 2048 rows.  e^-g overflows to infinity for
 // g < -88: the reciprocal is then 0 and the result -0, as it should be.
+// GATE_ACT (a constant of the build) chooses what the gated epilogues pass the gate through:
+// 0 silu; 1 the tanh form of gelu, 0.5 g (1 + tanh(a)) with a = sqrt(2/pi) (g + 0.044715 g^3),
+// which is g * sigmoid(2 a) and so the same two instructions.
+#ifndef GATE_ACT
+#define GATE_ACT 0
+#endif
 __device__ __forceinline__ float silu_f(float g) {
+#if GATE_ACT == 1
+  const float a2 = 1.5957691216057308f * (g + 0.044715f * g * g * g);
+  return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * a2));
+#else
   return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
+#endif
 }
 
 // Block = WAVES_M x WAVES_N waves, each owning (WM*32) x (WN*32) of the result as WM*WN

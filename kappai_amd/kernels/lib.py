@@ -26,7 +26,8 @@ GPU_ARCH = "gfx950"
 HIPCC_FLAGS = ["-O3", "-std=c++17", f"--offload-arch={GPU_ARCH}", "-shared", "-fPIC",
                "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
                "-Wno-unused-command-line-argument", "-Wno-pass-failed"]
-LIBRARIES = ["elementwise", "gemm", "shortconv", "attention", "sampling", "engine", "engine_api"]
+LIBRARIES = ["elementwise", "gemm", "shortconv", "attention", "sampling", "engine", "engine_api",
+             "groupnorm", "mingru", "diffattn", "moe"]
 # libraries made of more sources than the one of their own name
 EXTRA_SOURCES = {"engine": ["engine_parts"]}
 
@@ -45,7 +46,8 @@ def _python_flags() -> List[str]:
 # flags of single libraries beside HIPCC_FLAGS: name -> function that returns them
 EXTRA_FLAGS = {"engine_api": _python_flags}
 # libraries compiled once per value of a constant: name -> (constant, values built ahead)
-VARIANT_LIBRARIES = {"attention_mfma": ("HEAD_DIM", [16, 32, 48, 64, 80, 128, 256])}
+VARIANT_LIBRARIES = {"attention_mfma": ("HEAD_DIM", [16, 32, 48, 64, 80, 128, 256]),
+                     "gemm": ("GATE_ACT", [1])}
 
 
 class KernelBuildError(RuntimeError):

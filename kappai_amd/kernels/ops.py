@@ -580,11 +580,13 @@ def _out_in_fragment_order(wanted: bool, M: int, N: int, force_kernel: int) -> b
 
 
 def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0,
-                  weight_frag: Optional[torch.Tensor] = None, out_fragment: bool = False):
+                  weight_frag: Optional[torch.Tensor] = None, out_fragment: bool = False,
+                  activation: int = 0):
     """``silu(x Wg^T) * (x Wu^T)`` in one kernel: ``weight`` [2F, K] holds the gate and up
     matrices interleaved by ``interleave_gate_up``; bfloat16 only.  Returns [M, F].  ``x`` may
     be ``ScaledRows`` or ``FragmentRows``.  ``out_fragment``: with 8 to 16 rows the result may
-    come back as ``FragmentRows`` for the product that follows."""
+    come back as ``FragmentRows`` for the product that follows.  ``activation``: ``GLU_SILU`` (0)
+    or ``GLU_GELU_TANH`` (1) in place of silu; the product kernels are built once per gate."""
     scale = None
     if isinstance(x, ScaledRows):
         if (force_kernel not in (0, 2) or weight.dtype != BF16 or weight.dim() != 2
@@ -616,7 +618,8 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor, force_kernel: int = 0,
                   "and the tensors 16-byte aligned")
     c_frag = _out_in_fragment_order(out_fragment, M, F, force_kernel)
     out = torch.empty((16 if c_frag else M, F), dtype=BF16, device=x.device)
-    check(library("gemm").kappai_gemm_bf16_swiglu(
+    gemm = library("gemm") if not activation else library("gemm", GATE_ACT=int(activation))
+    check(gemm.kappai_gemm_bf16_swiglu(
         _ptr(x), *_matrix(weight, weight_frag), _ptr(out), _c_int(M), _c_int(F), _c_int(K),
         _c_int(lda), _c_int(F),
         _c_int(force_kernel), _c_int(a_frag),
@@ -1142,3 +1145,311 @@ def history_append(chosen: torch.Tensor, rows: torch.Tensor, slots: torch.Tensor
     check(library("sampling").kappai_history_append(
         _ptr(chosen), _ptr(rows), _ptr(slots), _ptr(history), _ptr(seen), _c_int(n),
         _c_int(history.shape[1]), _stream()), "history_append")
+
+
+# ---------------------------------------------------------------------------------------
+# grouped RMS norm, the input convolution of a sublayer, scaled embedding with positions
+# ---------------------------------------------------------------------------------------
+def add_group_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor,
+                      eps: float, groups: int, out_dtype, rows: Optional[torch.Tensor] = None,
+                      write_resid: bool = True) -> torch.Tensor:
+    """``resid += delta`` in float32 (``delta``: [T, D] bfloat16 or float32, float32 partial sums
+    [S, T, D] added in order, or None), then every one of ``groups`` equal consecutive parts of a
+    row divided by ``sqrt(mean(part^2) + eps)`` and the row multiplied by ``weight``.  With
+    ``rows`` only those rows are normalised and the residual is left alone.  Returns [n, D] in
+    ``out_dtype``."""
+    _gpu("resid", resid, F32)
+    _gpu("weight", weight, F32)
+    T, D = resid.shape
+    _need(weight.shape == (D,) and groups >= 1 and D % groups == 0,
+          lambda: f"add_group_rmsnorm: a width of {D} in {groups} groups, weight "
+                  f"{tuple(weight.shape)}")
+    _need((D + groups) * 4 <= 64 * 1024, lambda: f"add_group_rmsnorm: a width of {D} is beyond "
+          "what the kernel keeps of a row")
+    kind, n_part = 0, 0
+    if delta is not None:
+        _gpu("delta", delta, (F32, BF16))
+        if delta.dim() == 3:
+            _need(delta.dtype == F32 and tuple(delta.shape[1:]) == (T, D),
+                  lambda: f"add_group_rmsnorm: partial sums {tuple(delta.shape)}")
+            kind, n_part = 2, delta.shape[0]
+        else:
+            _need(tuple(delta.shape) == (T, D), lambda: f"add_group_rmsnorm: delta "
+                  f"{tuple(delta.shape)} for a residual {tuple(resid.shape)}")
+            kind, n_part = (1, 0) if delta.dtype == BF16 else (2, 1)
+        _need(rows is None, "add_group_rmsnorm: a pending update and a choice of rows")
+    n = T
+    if rows is not None:
+        _gpu("rows", rows, I32)
+        n = rows.shape[0]
+    out = torch.empty((n, D), dtype=out_dtype, device=resid.device)
+    check(library("groupnorm").kappai_add_group_rmsnorm(
+        _ptr(resid), _ptr(delta), _c_int(kind), _c_int(n_part), _c_int(T), _c_int(D),
+        _ptr(weight), _c_float(eps), _c_int(groups), _ptr(rows), _c_int(n), _ptr(out),
+        _c_int(_is_bf16(out_dtype)), _c_int(1 if write_resid and rows is None else 0),
+        _stream()), "add_group_rmsnorm")
+    return out
+
+
+CANON_MAX_TAPS = 16
+
+
+def canon_conv(h: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, row_pos: torch.Tensor,
+               row_seg: torch.Tensor, seg_start: torch.Tensor, seg_slot: torch.Tensor,
+               out_dtype) -> torch.Tensor:
+    """``h + conv(h)`` for float32 rows ``h`` [T, D]: ``conv(h)[t] = sum_j taps[:, j] *
+    h[t - n + 1 + j]`` along each request's sequence, inputs before the step's rows taken from
+    ``state`` [slots, n - 1, D] (the request's last n - 1 inputs, oldest first), zeros before
+    position 0.  The state is brought up to date.  Returns [T, D] in ``out_dtype``."""
+    _gpu("h", h, F32)
+    _gpu("taps", taps, F32)
+    _gpu("state", state, F32)
+    T, D = h.shape
+    n = taps.shape[1]
+    _need(taps.shape[0] == D and 1 <= n <= CANON_MAX_TAPS,
+          lambda: f"canon_conv: taps {tuple(taps.shape)} for a width of {D} (at most "
+                  f"{CANON_MAX_TAPS} taps)")
+    _need(state.dim() == 3 and tuple(state.shape[1:]) == (max(n - 1, 0), D),
+          lambda: f"canon_conv: state {tuple(state.shape)} is not [slots, {n - 1}, {D}]")
+    for name, t in (("row_pos", row_pos), ("row_seg", row_seg), ("seg_start", seg_start),
+                    ("seg_slot", seg_slot)):
+        _gpu(name, t, I32)
+    S = seg_slot.shape[0]
+    _need(row_pos.shape[0] == T and row_seg.shape[0] == T and seg_start.shape[0] == S + 1,
+          "canon_conv: row tables do not fit the batch")
+    out = torch.empty((T, D), dtype=out_dtype, device=h.device)
+    check(library("groupnorm").kappai_canon_conv(
+        _ptr(h), _ptr(taps), _ptr(state), _ptr(row_pos), _ptr(row_seg), _ptr(seg_start),
+        _ptr(seg_slot), _c_int(T), _c_int(S), _c_int(D), _c_int(n), _ptr(out),
+        _c_int(_is_bf16(out_dtype)), _stream()), "canon_conv")
+    return out
+
+
+def scale_add_positions(x: torch.Tensor, scale: float, table: torch.Tensor,
+                        row_pos: torch.Tensor) -> None:
+    """``x[t] = x[t] * scale + table[row_pos[t]]`` in place on float32 rows."""
+    _gpu("x", x, F32)
+    _gpu("table", table, (F32, BF16))
+    _gpu("row_pos", row_pos, I32)
+    T, D = x.shape
+    _need(table.dim() == 2 and table.shape[1] == D and row_pos.shape[0] == T,
+          lambda: f"scale_add_positions: x {tuple(x.shape)}, table {tuple(table.shape)}")
+    check(library("groupnorm").kappai_scale_add_positions(
+        _ptr(x), _c_float(scale), _ptr(table), _c_int(_is_bf16(table.dtype)), _ptr(row_pos),
+        _c_int(T), _c_int(D), _stream()), "scale_add_positions")
+
+
+GLU_SILU, GLU_GELU_TANH = 0, 1
+
+
+def glu(gate_up: torch.Tensor, kind: int) -> torch.Tensor:
+    """``act(gate_up[:, :F]) * gate_up[:, F:]`` for a fused [T, 2F] projection; ``kind``:
+    ``GLU_SILU`` or ``GLU_GELU_TANH`` (0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))))."""
+    _gpu("gate_up", gate_up, (F32, BF16))
+    _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0, "glu: [T, 2F] is needed")
+    _need(kind in (GLU_SILU, GLU_GELU_TANH), lambda: f"glu: unknown activation {kind}")
+    T, F = gate_up.shape[0], gate_up.shape[1] // 2
+    out = torch.empty((T, F), dtype=gate_up.dtype, device=gate_up.device)
+    check(library("elementwise").kappai_glu(
+        _ptr(gate_up), _ptr(out), _c_int(T), _c_int(F), _c_int(_is_bf16(gate_up.dtype)),
+        _c_int(kind), _stream()), "glu")
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+# minGRU
+# ---------------------------------------------------------------------------------------
+def mingru_chunk_rows() -> int:
+    return int(library("mingru").kappai_mingru_chunk_rows())
+
+
+def mingru_scan(proj: torch.Tensor, state: torch.Tensor, seg_start: torch.Tensor,
+                seg_pos0: torch.Tensor, seg_slot: torch.Tensor, out_dtype,
+                chunks: Optional[torch.Tensor] = None,
+                seg_chunk0: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """The minGRU recurrence over float32 projections [T, 3W] = (update gate | candidate | output
+    gate, biases added): ``S = (1 - z) S + z c`` with ``z = sigmoid``, ``c = u + 1/2`` for
+    ``u >= 0`` and ``sigmoid(u)`` below, output ``S * silu(g)`` [T, W] in ``out_dtype``.  ``state``
+    [slots, W] float32 is read (unless the segment starts at position 0) and left at the
+    segment's last row.  ``chunks`` [n, 3] = (segment, first row, rows) with ``seg_chunk0`` [S + 1]:
+    long segments are scanned chunk by chunk in three passes."""
+    _gpu("proj", proj, F32)
+    _gpu("state", state, F32)
+    T = proj.shape[0]
+    _need(proj.dim() == 2 and proj.shape[1] % 3 == 0, lambda: f"mingru_scan: {tuple(proj.shape)}")
+    W = proj.shape[1] // 3
+    _need(state.dim() == 2 and state.shape[1] == W,
+          lambda: f"mingru_scan: state {tuple(state.shape)} for a width of {W}")
+    for name, t in (("seg_start", seg_start), ("seg_pos0", seg_pos0), ("seg_slot", seg_slot)):
+        _gpu(name, t, I32)
+    S = seg_slot.shape[0]
+    _need(seg_start.shape[0] == S + 1 and seg_pos0.shape[0] == S,
+          "mingru_scan: segment tables do not fit")
+    out = torch.empty((T, W), dtype=out_dtype, device=proj.device)
+    n_chunks, carry = 0, None
+    if chunks is not None:
+        _gpu("chunks", chunks, I32)
+        _gpu("seg_chunk0", seg_chunk0, I32)
+        _need(chunks.dim() == 2 and chunks.shape[1] == 3 and seg_chunk0.shape[0] == S + 1,
+              "mingru_scan: chunk tables do not fit")
+        n_chunks = chunks.shape[0]
+        carry = torch.empty((n_chunks, 2, W), dtype=F32, device=proj.device)
+    check(library("mingru").kappai_mingru_scan(
+        _ptr(proj), _ptr(state), _ptr(seg_start), _ptr(seg_pos0), _ptr(seg_slot), _c_int(T),
+        _c_int(S), _c_int(W), _ptr(chunks), _ptr(seg_chunk0), _c_int(n_chunks), _ptr(carry),
+        _ptr(out), _c_int(_is_bf16(out_dtype)), _stream()), "mingru_scan")
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+# differential attention: the two maps of a head as heads of the paged attention kernels
+# ---------------------------------------------------------------------------------------
+def diff_store(proj: torch.Tensor, n_heads: int, n_kv_heads: int, dim: int, vdim: int,
+               head_size: int, k_pool: torch.Tensor, v_pool: torch.Tensor, row_pos: torch.Tensor,
+               row_seg: torch.Tensor, block_tables: torch.Tensor, page_size: int,
+               store_kv: bool = True) -> torch.Tensor:
+    """From ``proj`` [T, H 2 dim + G 2 dim + G vdim] (a head's two maps side by side): queries
+    [T, 2H head_size] with map (h, m) of head h = g R + i as head (2 g + m) R + i, widened with
+    zeros; keys of map m of kv head g stored as kv head 2 g + m of pools made for 2G kv heads of
+    ``head_size``, the kv head's values under both."""
+    H, G, d, dv, D = n_heads, n_kv_heads, dim, vdim, head_size
+    _gpu("proj", proj, (F32, BF16), contiguous=False)
+    T = proj.shape[0]
+    need = (H * 2 * d + G * 2 * d + G * dv) if store_kv else H * 2 * d
+    _need(proj.dim() == 2 and proj.shape[1] >= need and proj.stride(1) == 1,
+          lambda: f"diff_store: proj {tuple(proj.shape)} holds fewer than {need} columns")
+    _need(H % G == 0 and d <= D and dv <= D, lambda: f"diff_store: {H} heads over {G}, sizes "
+          f"{d} and {dv} in heads of {D}")
+    _gpu("row_pos", row_pos, I32)
+    _gpu("row_seg", row_seg, I32)
+    max_blocks = 0
+    if store_kv:
+        _gpu("k_pool", k_pool, proj.dtype)
+        _gpu("v_pool", v_pool, proj.dtype)
+        _gpu("block_tables", block_tables, I32)
+        _check_pools(k_pool, v_pool, 2 * G, page_size, D)
+        _need(block_tables.dim() == 2, "block_tables must be [segments, max_blocks]")
+        max_blocks = block_tables.shape[1]
+    q = torch.empty((T, 2 * H * D), dtype=proj.dtype, device=proj.device)
+    check(library("diffattn").kappai_diff_store(
+        _ptr(proj), _c_int(proj.stride(0)), _ptr(q), _ptr(k_pool), _ptr(v_pool), _ptr(row_pos),
+        _ptr(row_seg), _ptr(block_tables if store_kv else None), _c_int(max_blocks), _c_int(T),
+        _c_int(H), _c_int(G), _c_int(d), _c_int(dv), _c_int(D), _c_int(page_size),
+        _c_int(1 if store_kv else 0), _c_int(_is_bf16(proj.dtype)), _stream()), "diff_store")
+    return q
+
+
+def diff_combine(ctx: torch.Tensor, n_heads: int, n_kv_heads: int, vdim: int, head_size: int,
+                 lam: float, eps: float, gain: float) -> torch.Tensor:
+    """``o = a1 - lam * a2`` per head from the two maps' outputs ``ctx`` [T, 2H head_size] (in
+    ``diff_store``'s order), ``o / sqrt(mean(o^2) + eps) * gain`` over the head's ``vdim`` values.
+    Returns [T, H vdim]."""
+    H, G, dv, D = n_heads, n_kv_heads, vdim, head_size
+    _gpu("ctx", ctx, (F32, BF16))
+    T = ctx.shape[0]
+    _need(tuple(ctx.shape) == (T, 2 * H * D), lambda: f"diff_combine: ctx {tuple(ctx.shape)}")
+    out = torch.empty((T, H * dv), dtype=ctx.dtype, device=ctx.device)
+    check(library("diffattn").kappai_diff_combine(
+        _ptr(ctx), _ptr(out), _c_int(T), _c_int(H), _c_int(G), _c_int(dv), _c_int(D),
+        _c_float(lam), _c_float(eps), _c_float(gain), _c_int(_is_bf16(ctx.dtype)), _stream()),
+        "diff_combine")
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+# mixture of experts
+# ---------------------------------------------------------------------------------------
+MOE_MAX_TOP = 16
+
+
+def moe_route(x: torch.Tensor, router: torch.Tensor, top: int):
+    """Router logits ``x router^T`` in float32, the ``top`` largest of a row chosen (the lowest
+    index wins a tie), weights = softmax over the chosen logits.  Returns (experts [T, top] int32,
+    weights [T, top] float32), the largest first."""
+    _gpu("x", x, (F32, BF16), contiguous=False)
+    _gpu("router", router, F32)
+    T, D = x.shape
+    E = router.shape[0]
+    _need(router.shape == (E, D) and x.stride(1) == 1 and 1 <= top <= min(E, MOE_MAX_TOP),
+          lambda: f"moe_route: x {tuple(x.shape)}, router {tuple(router.shape)}, top {top}")
+    idx = torch.empty((T, top), dtype=I32, device=x.device)
+    wts = torch.empty((T, top), dtype=F32, device=x.device)
+    check(library("moe").kappai_moe_route(
+        _ptr(x), _c_int(x.stride(0)), _c_int(_is_bf16(x.dtype)), _ptr(router), _c_int(T),
+        _c_int(D), _c_int(E), _c_int(top), _ptr(idx), _ptr(wts), _stream()), "moe_route")
+    return idx, wts
+
+
+@dataclass
+class MoePlan:
+    """The step's (row, choice) pairs in expert order: ``slot_of_pair`` [T top], ``pair_of_slot``
+    [tiles * tile_rows] (-1: empty), ``tile_expert`` [tiles] (-1: unused)."""
+    slot_of_pair: torch.Tensor
+    pair_of_slot: torch.Tensor
+    tile_expert: torch.Tensor
+    n_tiles: int
+    tile_rows: int
+    top: int
+
+
+def moe_plan(experts: torch.Tensor, n_experts: int) -> MoePlan:
+    _gpu("experts", experts, I32)
+    T, top = experts.shape
+    P = T * top
+    tile = int(library("moe").kappai_moe_tile_rows())
+    n_tiles = P // tile + min(n_experts, P)
+    dev = experts.device
+    plan = MoePlan(torch.empty((P,), dtype=I32, device=dev),
+                   torch.empty((n_tiles * tile,), dtype=I32, device=dev),
+                   torch.empty((n_tiles,), dtype=I32, device=dev), n_tiles, tile, top)
+    check(library("moe").kappai_moe_plan(
+        _ptr(experts), _c_int(P), _c_int(n_experts), _c_int(n_tiles), _ptr(plan.slot_of_pair),
+        _ptr(plan.pair_of_slot), _ptr(plan.tile_expert), _stream()), "moe_plan")
+    return plan
+
+
+def moe_experts_gated(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor,
+                      plan: MoePlan) -> torch.Tensor:
+    """``silu(x Wg[e]^T) * (x Wu[e]^T)`` for every slot of the plan ([slots, F], the dtype of
+    ``x``; empty slots are left unwritten).  ``w_gate``, ``w_up``: [E, F, D]."""
+    _gpu("x", x, (F32, BF16), contiguous=False)
+    _gpu("w_gate", w_gate, x.dtype)
+    _gpu("w_up", w_up, x.dtype)
+    E, F, D = w_gate.shape
+    _need(w_up.shape == w_gate.shape and x.shape[1] == D and x.stride(1) == 1,
+          lambda: f"moe_experts_gated: x {tuple(x.shape)}, matrices {tuple(w_gate.shape)}")
+    out = torch.empty((plan.n_tiles * plan.tile_rows, F), dtype=x.dtype, device=x.device)
+    check(library("moe").kappai_moe_gemm(
+        _ptr(x), _c_int(x.stride(0)), _ptr(w_gate), _ptr(w_up), _c_int(F), _c_int(D),
+        _ptr(plan.tile_expert), _ptr(plan.pair_of_slot), _c_int(plan.top), _c_int(plan.n_tiles),
+        _ptr(out), _c_int(1), _c_int(_is_bf16(x.dtype)), _stream()), "moe_gemm (gate, up)")
+    return out
+
+
+def moe_experts_down(act: torch.Tensor, w_down: torch.Tensor, plan: MoePlan) -> torch.Tensor:
+    """``act W_down[e]^T`` for every slot of the plan: float32 [slots, D]."""
+    _gpu("act", act, (F32, BF16))
+    _gpu("w_down", w_down, act.dtype)
+    E, D, F = w_down.shape
+    _need(tuple(act.shape) == (plan.n_tiles * plan.tile_rows, F),
+          lambda: f"moe_experts_down: act {tuple(act.shape)}, matrices {tuple(w_down.shape)}")
+    out = torch.empty((act.shape[0], D), dtype=F32, device=act.device)
+    check(library("moe").kappai_moe_gemm(
+        _ptr(act), _c_int(F), _ptr(w_down), _vp(0), _c_int(D), _c_int(F),
+        _ptr(plan.tile_expert), _ptr(plan.pair_of_slot), _c_int(plan.top), _c_int(plan.n_tiles),
+        _ptr(out), _c_int(0), _c_int(_is_bf16(act.dtype)), _stream()), "moe_gemm (down)")
+    return out
+
+
+def moe_combine(y: torch.Tensor, weights: torch.Tensor, plan: MoePlan) -> torch.Tensor:
+    """``out[t] = sum_k weights[t, k] * y[slot of (t, k)]`` in the order of k: float32 [T, D]."""
+    _gpu("y", y, F32)
+    _gpu("weights", weights, F32)
+    T, top = weights.shape
+    D = y.shape[1]
+    _need(top == plan.top and plan.slot_of_pair.shape[0] == T * top, "moe_combine: another plan")
+    out = torch.empty((T, D), dtype=F32, device=y.device)
+    check(library("moe").kappai_moe_combine(
+        _ptr(y), _ptr(plan.slot_of_pair), _ptr(weights), _c_int(T), _c_int(top), _c_int(D),
+        _ptr(out), _stream()), "moe_combine")
+    return out

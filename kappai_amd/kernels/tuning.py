@@ -63,3 +63,10 @@ FUSED_QK_MAX_ROWS = 4
 # 63 rows of at most 2300 keys beside portions of 512 rows the two kernels took 49 us a layer where
 # the tiled kernel alone took 43, hence not from 1024 on.
 LONE_ROWS_FROM = 4096
+
+# The minGRU recurrence over a segment: one thread a channel walks the rows in order, which is the
+# whole of a decode step and fine for short portions; a segment of more than SCAN_CHUNKS_FROM_ROWS
+# rows is cut into chunks of SCAN_CHUNK_ROWS rows that are scanned side by side in three passes
+# (chunk sums, carry over the chunks, outputs).
+SCAN_CHUNK_ROWS = 32
+SCAN_CHUNKS_FROM_ROWS = 64

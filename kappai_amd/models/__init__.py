@@ -7,6 +7,7 @@ import torch
 
 from ..config.base import ModelConfig, load_config, lookup_architecture
 from ..weights.loader import check_and_load, parse_dtype
+from . import dapipel  # noqa: F401  (registers Dapipel)
 from . import lfm2  # noqa: F401  (registers Lfm2ForCausalLM)
 from .base import LayerCall, Model
 

@@ -1,11 +1,17 @@
 from .attention import GroupedQueryAttention
 from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Block, FeedForward,
                    Hidden, Mixer, Norm, Part, PositionEncoding, make_part, register_part)
-from .block import PreNormBlock
+from .block import ConvInputBlock, PreNormBlock
+from .diff_attention import DifferentialAttention
 from .embedding import OutputHead, TokenEmbedding
 from .feed_forward import SwiGLU
+from .group_norm import GroupRMSNorm
+from .input_conv import ShortInputConv
 from .linear import Linear
+from .mingru import MinGRU
+from .moe import MixtureOfExperts
 from .norm import RMSNorm
+from .positions import LearnedPositions
 from .rotary import RotaryEncoding, Rotation
 from .shortconv import GatedShortConv
 
@@ -13,4 +19,5 @@ __all__ = ["GroupedQueryAttention", "BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS"
            "POSITION_ENCODINGS", "Block", "FeedForward", "Hidden", "Mixer", "Norm", "Part",
            "PositionEncoding", "make_part", "register_part", "PreNormBlock", "OutputHead",
            "TokenEmbedding", "SwiGLU", "Linear", "RMSNorm", "RotaryEncoding", "Rotation",
-           "GatedShortConv"]
+           "GatedShortConv", "ConvInputBlock", "DifferentialAttention", "GroupRMSNorm",
+           "ShortInputConv", "MinGRU", "MixtureOfExperts", "LearnedPositions"]

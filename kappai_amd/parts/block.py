@@ -125,3 +125,77 @@ class PreNormBlock(Block):
 
 
 register_part("block", "pre_norm", PreNormBlock)
+
+
+class ConvInputBlock(Block):
+    """``x += mixer(conv(norm(x))); x += feed_forward(conv(norm(x)))``: the pre-norm arrangement
+    with a short causal convolution (``parts.input_conv.ShortInputConv``) between each norm and
+    the sublayer that reads it.  The norm hands the convolution float32 rows; the convolution
+    rounds to the compute dtype once.  ``feed_forward`` (with its norm and convolution) may be
+    None: the layer is then its mixer alone.  The block's cache is a bundle: the mixer's own need
+    under "mixer" and the convolutions' histories under "mixer_conv" and "ffn_conv"."""
+
+    def __init__(self, mixer_norm: Norm, mixer_conv, mixer: Mixer, ffn_norm=None, ffn_conv=None,
+                 feed_forward=None):
+        self.mixer_norm, self.mixer_conv, self.mixer = mixer_norm, mixer_conv, mixer
+        self.ffn_norm, self.ffn_conv, self.feed_forward = ffn_norm, ffn_conv, feed_forward
+        if (feed_forward is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+
+    def _parts(self):
+        return tuple(p for p in (self.mixer_norm, self.mixer_conv, self.mixer, self.ffn_norm,
+                                 self.ffn_conv, self.feed_forward) if p is not None)
+
+    @property
+    def capturable(self) -> bool:
+        return all(p.capturable for p in self._parts())
+
+    @property
+    def step_tables(self):
+        return [t for t in (p.step_tables for p in self._parts()) if t is not None]
+
+    def cache_spec(self):
+        from ..cache.specs import CacheBundle
+        members = [("mixer", self.mixer.cache_spec())]
+        if self.mixer_conv is not None:
+            members.append(("mixer_conv", self.mixer_conv.cache_spec()))
+        if self.ffn_conv is not None:
+            members.append(("ffn_conv", self.ffn_conv.cache_spec()))
+        return CacheBundle(tuple(members))
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s for p in self._parts() for s in p.tensor_specs()]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for p in self._parts():
+            p.bind(tensors)
+
+    @staticmethod
+    def _read(norm, conv, resid, delta, batch, state):
+        delta = summed_delta(norm, delta)
+        if conv is None:
+            return norm.add_norm(resid, delta)
+        if getattr(norm, "takes_out_dtype", False):
+            h = norm.add_norm(resid, delta, out_dtype=torch.float32)
+        else:
+            h = ops.cast(norm.add_norm(resid, delta), torch.float32)
+        return conv.forward(h, batch, state)
+
+    def forward(self, h: Hidden, batch, cache, shared_cache: bool = False) -> Hidden:
+        if shared_cache:
+            raise ValueError("the input convolutions' histories cannot be read by another layer")
+        resid = h.resid
+        x = self._read(self.mixer_norm, self.mixer_conv, resid, h.delta, batch,
+                       cache.parts.get("mixer_conv"))
+        mixed = self.mixer.forward(x, batch, cache.part("mixer"))
+        if self.feed_forward is None:
+            return Hidden(resid, mixed)
+        x = self._read(self.ffn_norm, self.ffn_conv, resid, mixed, batch,
+                       cache.parts.get("ffn_conv"))
+        return Hidden(resid, self.feed_forward.forward(x, batch))
+
+    def weight_bytes(self) -> int:
+        return sum(p.weight_bytes() for p in self._parts())
+
+
+register_part("block", "conv_input", ConvInputBlock)

@@ -15,15 +15,17 @@ class TokenEmbedding(Part):
     """Rows of the table widened to float32, without a scale
     (kappai: src/recipe/scratch.c:195-235)."""
 
-    def __init__(self, name: str, vocab: int, width: int):
+    def __init__(self, name: str, vocab: int, width: int, suffix: str = ".weight"):
+        """``suffix``: how the table's tensor name ends in the checkpoint."""
         self.name, self.vocab, self.width = name, vocab, width
+        self.tensor_name = name + suffix
         self.table: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [TensorSpec(self.name + ".weight", (self.vocab, self.width), TABLE, INIT_NORMAL)]
+        return [TensorSpec(self.tensor_name, (self.vocab, self.width), TABLE, INIT_NORMAL)]
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.table = tensors[self.name + ".weight"]
+        self.table = tensors[self.tensor_name]
 
     def forward(self, tokens: torch.Tensor) -> torch.Tensor:
         with profile.scope("embd"):
@@ -41,8 +43,9 @@ class OutputHead(Part):
     """Logits in float32 for the rows asked for.  When tied the head is the embedding
     table itself (kappai: src/model.c:2562-2571)."""
 
-    def __init__(self, name: str, vocab: int, width: int, tied_to: Optional[TokenEmbedding]):
-        self.linear = Linear([name], width, [vocab], stage="logits_matmul")
+    def __init__(self, name: str, vocab: int, width: int, tied_to: Optional[TokenEmbedding],
+                 suffix: str = ".weight"):
+        self.linear = Linear([name], width, [vocab], stage="logits_matmul", weight_suffix=suffix)
         self.tied_to = tied_to
 
     def tensor_specs(self) -> List[TensorSpec]:

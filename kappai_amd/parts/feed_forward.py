@@ -27,14 +27,24 @@ class SwiGLU(FeedForward):
     takes_deferred_rows = True     # its first product takes what ops.linear takes
     adds_residual = True           # its last product can add into the residual stream
 
-    def __init__(self, prefix: str, width: int, hidden: int, dtype: torch.dtype, names=None):
+    ACTIVATIONS = {"silu": ops.GLU_SILU, "gelu_tanh": ops.GLU_GELU_TANH}
+
+    def __init__(self, prefix: str, width: int, hidden: int, dtype: torch.dtype, names=None,
+                 activation: str = "silu", weight_suffix: str = ".weight"):
+        """``activation``: what the gate passes through, "silu" or "gelu_tanh" (the tanh form of
+        GELU): ``W_down (act(W_gate x) * W_up x)``."""
         n = {"gate": "w1", "up": "w3", "down": "w2"}
         n.update(names or {})
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"unknown gate activation {activation!r}; known: "
+                             f"{', '.join(self.ACTIVATIONS)}")
         self.width, self.hidden, self.dtype = width, hidden, dtype
+        self.activation = activation
         self.fused = False
         self.gate_up = Linear([prefix + n["gate"], prefix + n["up"]], width, [hidden, hidden],
-                              stage="matmul_ffn_gate_up")
-        self.down = Linear([prefix + n["down"]], hidden, [width], stage="matmul_ffn_down")
+                              stage="matmul_ffn_gate_up", weight_suffix=weight_suffix)
+        self.down = Linear([prefix + n["down"]], hidden, [width], stage="matmul_ffn_down",
+                           weight_suffix=weight_suffix)
 
     def tensor_specs(self) -> List[TensorSpec]:
         return self.gate_up.tensor_specs() + self.down.tensor_specs()
@@ -52,16 +62,20 @@ class SwiGLU(FeedForward):
     def forward(self, x, batch, into=None):
         if self.fused and x.dtype == torch.bfloat16:
             with profile.scope("matmul_ffn_gate_up", self.gate_up.weight_bytes()):
-                act = ops.linear_swiglu(x, self.gate_up.weight, out_fragment=True)
+                act = ops.linear_swiglu(x, self.gate_up.weight, out_fragment=True,
+                                        activation=self.ACTIVATIONS[self.activation])
             return self.down.forward(act, partial_sums=True, add_into=into)
         gate_up = self.gate_up.forward(x)
         with profile.scope("ffn_act"):
-            act = ops.swiglu(gate_up)
+            act = (ops.swiglu(gate_up) if self.activation == "silu"
+                   else ops.glu(gate_up, self.ACTIVATIONS[self.activation]))
         return self.down.forward(act, partial_sums=True, add_into=into)
 
     def c_part(self, plan, view=None, shared_cache: bool = False):
         """The runner "feed_forward.swiglu" (csrc/engine_parts.hip) makes the same choices as
         ``forward``."""
+        if self.activation != "silu":
+            return None            # the runner on the C side knows the SiLU gate only
         first = plan.linear(self.gate_up)
         desc = SwiGLUDesc(first, plan.linear(self.down), self.hidden, 1 if self.fused else 0)
         return plan.part("feed_forward.swiglu", desc, takes_deferred_rows=True,

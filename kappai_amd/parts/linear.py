@@ -17,10 +17,20 @@ class Linear(Part):
     (kappai's optional load-time fusion of q,k,v and gate,up, src/model.c:930-948)."""
 
     def __init__(self, names: Sequence[str], in_features: int, out_features: Sequence[int],
-                 bias: bool = False, stage: str = "matmul", cut_rows_at: Sequence[int] = ()):
+                 bias=False, stage: str = "matmul", cut_rows_at: Sequence[int] = (),
+                 weight_suffix: str = ".weight", bias_suffix: str = ".bias"):
         """``cut_rows_at``: row counts at which the owner wants to use the first rows of the
-        stacked matrix by themselves (``first_rows``)."""
+        stacked matrix by themselves (``first_rows``).  ``bias``: whether the matrices have
+        biases, for all of them or one by one (the stacked bias is zero where a matrix has
+        none).  ``weight_suffix`` / ``bias_suffix``: how a checkpoint's tensor names end."""
         self.names = list(names)
+        self.weight_suffix, self.bias_suffix = weight_suffix, bias_suffix
+        self.bias_of = [bool(bias)] * len(self.names) if isinstance(bias, bool) else [
+            bool(b) for b in bias]
+        if len(self.bias_of) != len(self.names):
+            raise ValueError(f"{self.names}: {len(self.bias_of)} bias flags for "
+                             f"{len(self.names)} matrices")
+        bias = any(self.bias_of)
         self.cut_rows_at = list(cut_rows_at)
         self.stage = stage              # the row of the --time table this product is booked under
         self.in_features = in_features
@@ -35,16 +45,17 @@ class Linear(Part):
 
     def tensor_specs(self) -> List[TensorSpec]:
         specs = []
-        for n, o in zip(self.names, self.out_features):
-            specs.append(TensorSpec(n + ".weight", (o, self.in_features), MATRIX, INIT_NORMAL))
-            if self.has_bias:
-                specs.append(TensorSpec(n + ".bias", (o,), VECTOR, INIT_SMALL))
+        for n, o, b in zip(self.names, self.out_features, self.bias_of):
+            specs.append(TensorSpec(n + self.weight_suffix, (o, self.in_features), MATRIX,
+                                    INIT_NORMAL))
+            if b:
+                specs.append(TensorSpec(n + self.bias_suffix, (o,), VECTOR, INIT_SMALL))
         return specs
 
     def bind(self, tensors: Dict[str, torch.Tensor], arrange=None) -> None:
         """``arrange(matrix) -> matrix``: another order of the stacked rows that the owner's
         kernel wants (gate and up rows interleaved), or None to keep them as they are."""
-        ws = [tensors[n + ".weight"] for n in self.names]
+        ws = [tensors[n + self.weight_suffix] for n in self.names]
         if len({w.dtype for w in ws}) > 1:           # stored in different widths: widen
             ws = [w.to(torch.float32) for w in ws]
         weight = ws[0] if len(ws) == 1 else torch.cat(ws, dim=0).contiguous()
@@ -53,7 +64,9 @@ class Linear(Part):
             weight = weight if arranged is None else arranged
         self.set_weight(weight)
         if self.has_bias:
-            bs = [tensors[n + ".bias"].to(torch.float32) for n in self.names]
+            bs = [tensors[n + self.bias_suffix].to(torch.float32) if b
+                  else torch.zeros(o, dtype=torch.float32, device=ws[0].device)
+                  for n, o, b in zip(self.names, self.out_features, self.bias_of)]
             self.bias = bs[0] if len(bs) == 1 else torch.cat(bs, dim=0).contiguous()
 
     def set_weight(self, weight: torch.Tensor) -> None:

@@ -73,11 +73,15 @@ def interleave_gate_up(gate, up):
     return torch.cat([g, u], dim=1).reshape(2 * F, K).contiguous()
 
 
-def linear_swiglu(x, weight, force_kernel=0, weight_frag=None, out_fragment=False):
+def linear_swiglu(x, weight, force_kernel=0, weight_frag=None, out_fragment=False, activation=0):
     F = weight.shape[0] // 2
     y = (x.to(F32) @ weight.to(F32).T).reshape(x.shape[0], F // SWIGLU_GROUP, 2, SWIGLU_GROUP)
     g, u = y[:, :, 0, :].reshape(-1, F), y[:, :, 1, :].reshape(-1, F)
-    return (g / (1.0 + torch.exp(-g)) * u).to(x.dtype)
+    if activation == 1:
+        a = 0.5 * g * (1.0 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3)))
+    else:
+        a = g / (1.0 + torch.exp(-g))
+    return (a * u).to(x.dtype)
 
 
 def shortconv(proj, taps, bias, state, row_seg, seg_start, seg_pos0, seg_slot):
@@ -248,7 +252,154 @@ def history_append(chosen, rows, slots, history, seen):
         seen[slot] += 1
 
 
-ALL = ["embed_rows", "add_rmsnorm", "add_residual", "sum_partial_sums", "swiglu", "cast", "linear", "linear_swiglu",
+
+# ---- grouped norm, input convolution, positions -------------------------------------------
+def add_group_rmsnorm(resid, delta, weight, eps, groups, out_dtype, rows=None, write_resid=True):
+    x = resid
+    if delta is not None:
+        parts = delta if delta.dim() == 3 else delta[None]
+        for p in parts:
+            x = x + p.to(F32)
+        if write_resid and rows is None:
+            resid.copy_(x)
+    if rows is not None:
+        x = x[rows.long()]
+    n, D = x.shape
+    g = x.reshape(n, groups, D // groups)
+    g = g * (1.0 / torch.sqrt((g * g).mean(dim=-1, keepdim=True) + eps))
+    return (g.reshape(n, D) * weight).to(out_dtype)
+
+
+def canon_conv(h, taps, state, row_pos, row_seg, seg_start, seg_slot, out_dtype):
+    T, D = h.shape
+    n = taps.shape[1]
+    out = h.clone()
+    for t in range(T):
+        s = int(row_seg[t])
+        local = t - int(seg_start[s])
+        slot = int(seg_slot[s])
+        for j in range(n):
+            back = n - 1 - j
+            if int(row_pos[t]) - back < 0:
+                continue
+            v = h[t - back] if local - back >= 0 else state[slot, n - 1 + local - back]
+            out[t] += taps[:, j] * v
+    for s in range(seg_slot.shape[0]):
+        first, last = int(seg_start[s]), int(seg_start[s + 1])
+        slot = int(seg_slot[s])
+        hist = torch.cat([state[slot], h[first:last]], dim=0)
+        state[slot] = hist[hist.shape[0] - (n - 1):]
+    return out.to(out_dtype)
+
+
+def scale_add_positions(x, scale, table, row_pos):
+    x.mul_(scale).add_(table[row_pos.long()].to(F32))
+
+
+def glu(gate_up, kind):
+    F = gate_up.shape[1] // 2
+    g, u = gate_up[:, :F].to(F32), gate_up[:, F:].to(F32)
+    if kind == 1:
+        a = 0.5 * g * (1.0 + torch.tanh(0.7978845608028654 * (g + 0.044715 * g ** 3)))
+    else:
+        a = g / (1.0 + torch.exp(-g))
+    return (a * u).to(gate_up.dtype)
+
+
+# ---- minGRU ----------------------------------------------------------------------------------
+def mingru_scan(proj, state, seg_start, seg_pos0, seg_slot, out_dtype, chunks=None,
+                seg_chunk0=None):
+    T, W = proj.shape[0], proj.shape[1] // 3
+    out = torch.empty((T, W), dtype=F32)
+    for s in range(seg_slot.shape[0]):
+        slot = int(seg_slot[s])
+        S = state[slot].clone() if int(seg_pos0[s]) > 0 else torch.zeros(W)
+        for t in range(int(seg_start[s]), int(seg_start[s + 1])):
+            z = torch.sigmoid(proj[t, :W])
+            u = proj[t, W:2 * W]
+            c = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
+            S = (1.0 - z) * S + z * c
+            g = proj[t, 2 * W:]
+            out[t] = S * (g * torch.sigmoid(g))
+        state[slot] = S
+    return out.to(out_dtype)
+
+
+# ---- differential attention -------------------------------------------------------------------
+def diff_store(proj, n_heads, n_kv_heads, dim, vdim, head_size, k_pool, v_pool, row_pos, row_seg,
+               block_tables, page_size, store_kv=True):
+    H, G, d, dv, D = n_heads, n_kv_heads, dim, vdim, head_size
+    T, R = proj.shape[0], n_heads // n_kv_heads
+    q = torch.zeros((T, 2 * H, D), dtype=proj.dtype)
+    qs = proj[:, :H * 2 * d].reshape(T, G, R, 2, d)
+    q.view(T, G, 2, R, D)[..., :d] = qs.permute(0, 1, 3, 2, 4)
+    if store_kv:
+        ks = proj[:, H * 2 * d:(H + G) * 2 * d].reshape(T, 2 * G, d)
+        vs = proj[:, (H + G) * 2 * d:(H + G) * 2 * d + G * dv].reshape(T, G, dv)
+        for t in range(T):
+            p = int(row_pos[t])
+            page = int(block_tables[int(row_seg[t]), p // page_size])
+            assert page >= 0, "a key is stored into a page that was given back"
+            k_pool[page, :, p % page_size, :] = 0
+            k_pool[page, :, p % page_size, :d] = ks[t]
+            v_pool[page, :, :, p % page_size] = 0
+            v_pool[page, :, :dv, p % page_size] = vs[t].repeat_interleave(2, dim=0)
+    return q.reshape(T, 2 * H * D)
+
+
+def diff_combine(ctx, n_heads, n_kv_heads, vdim, head_size, lam, eps, gain):
+    H, G, dv, D = n_heads, n_kv_heads, vdim, head_size
+    T, R = ctx.shape[0], n_heads // n_kv_heads
+    a = ctx.to(F32).reshape(T, G, 2, R, D)[..., :dv]
+    o = a[:, :, 0] - lam * a[:, :, 1]                      # [T, G, R, dv]
+    o = o * (gain / torch.sqrt((o * o).mean(dim=-1, keepdim=True) + eps))
+    return o.reshape(T, H * dv).to(ctx.dtype)
+
+
+# ---- mixture of experts -----------------------------------------------------------------------
+class _Plan:
+    def __init__(self, experts):
+        self.experts = experts
+
+
+def moe_route(x, router, top):
+    logits = x.to(F32) @ router.T
+    best, chosen = torch.topk(logits, top, dim=-1)
+    return chosen.to(torch.int32), torch.softmax(best, dim=-1)
+
+
+def moe_plan(experts, n_experts):
+    return _Plan(experts)
+
+
+def moe_experts_gated(x, w_gate, w_up, plan):
+    T, top = plan.experts.shape
+    out = torch.empty((T, top, w_gate.shape[1]), dtype=x.dtype)
+    for t in range(T):
+        for k in range(top):
+            e = int(plan.experts[t, k])
+            g = w_gate[e].to(F32) @ x[t].to(F32)
+            u = w_up[e].to(F32) @ x[t].to(F32)
+            out[t, k] = (g / (1.0 + torch.exp(-g)) * u).to(x.dtype)
+    return out
+
+
+def moe_experts_down(act, w_down, plan):
+    T, top = plan.experts.shape
+    out = torch.empty((T, top, w_down.shape[1]), dtype=F32)
+    for t in range(T):
+        for k in range(top):
+            out[t, k] = w_down[int(plan.experts[t, k])].to(F32) @ act[t, k].to(F32)
+    return out
+
+
+def moe_combine(y, weights, plan):
+    return (y * weights[:, :, None]).sum(dim=1)
+
+
+ALL = ["add_group_rmsnorm", "canon_conv", "scale_add_positions", "glu", "mingru_scan", "diff_store",
+       "diff_combine", "moe_route", "moe_plan", "moe_experts_gated", "moe_experts_down", "moe_combine",
+       "embed_rows", "add_rmsnorm", "add_residual", "sum_partial_sums", "swiglu", "cast", "linear", "linear_swiglu",
        "interleave_gate_up", "shortconv", "linear_shortconv_step",
        "qk_norm_rope_store", "paged_attention", "sample_rows", "sample_filtered",
        "repeat_penalty", "history_set", "repeat_penalty_history", "history_append"]
