@@ -1156,8 +1156,8 @@ def add_group_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight
     """``resid += delta`` in float32 (``delta``: [T, D] bfloat16 or float32, float32 partial sums
     [S, T, D] added in order, or None), then every one of ``groups`` equal consecutive parts of a
     row divided by ``sqrt(mean(part^2) + eps)`` and the row multiplied by ``weight``.  With
-    ``rows`` only those rows are normalised and the residual is left alone.  Returns [n, D] in
-    ``out_dtype``."""
+    ``rows`` only those rows are summed and normalised and the residual is left alone.  Returns
+    [n, D] in ``out_dtype``."""
     _gpu("resid", resid, F32)
     _gpu("weight", weight, F32)
     T, D = resid.shape
@@ -1177,7 +1177,6 @@ def add_group_rmsnorm(resid: torch.Tensor, delta: Optional[torch.Tensor], weight
             _need(tuple(delta.shape) == (T, D), lambda: f"add_group_rmsnorm: delta "
                   f"{tuple(delta.shape)} for a residual {tuple(resid.shape)}")
             kind, n_part = (1, 0) if delta.dtype == BF16 else (2, 1)
-        _need(rows is None, "add_group_rmsnorm: a pending update and a choice of rows")
     n = T
     if rows is not None:
         _gpu("rows", rows, I32)
