@@ -74,7 +74,8 @@ def differential_attention(h, t, p, m: dict, eps: float, rounding=None):
     are not seen."""
     T = h.shape[0]
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    window, scale, diff = m["mask"]["size"], m["scale"], m["diff"]
+    window = m["mask"]["size"] if m.get("mask") else T + 1
+    scale, diff = m["scale"], m["diff"]
     q = _r(matmul(h, t[p + "q"], rounding), rounding).reshape(T, H, 2, d)
     k = _r(matmul(h, t[p + "k"], rounding), rounding).reshape(T, G, 2, d)
     v = _r(matmul(h, t[p + "v"], rounding), rounding).reshape(T, G, dv)
@@ -96,19 +97,27 @@ def differential_attention(h, t, p, m: dict, eps: float, rounding=None):
     return matmul(out.reshape(T, H * dv), t[p + "o"], rounding)
 
 
-def mingru(h, t, p, rounding=None, state: Optional[torch.Tensor] = None):
-    """``S_t = (1 - z_t) S_(t-1) + z_t c_t`` from a zero state; ``c = u + 1/2`` where ``u >= 0``,
-    ``sigmoid(u)`` below; the output is ``W_o (S_t * silu(W_g h))``."""
-    z = torch.sigmoid(matmul(h, t[p + "z"], rounding) + t[p + "z.b"].to(F64))
-    u = matmul(h, t[p + "x"], rounding) + t[p + "x.b"].to(F64)
-    cand = torch.where(u >= 0, u + 0.5, torch.sigmoid(u))
-    gate = silu(matmul(h, t[p + "g"], rounding))
+def mingru_recurrence(pz, pu, pg, state: Optional[torch.Tensor] = None):
+    """From the three projections (biases added): the gated states times the output gate
+    [T, W], and the last state."""
+    z = torch.sigmoid(pz)
+    cand = torch.where(pu >= 0, pu + 0.5, torch.sigmoid(pu))
+    gate = silu(pg)
     S = torch.zeros(z.shape[1], dtype=F64) if state is None else state.clone()
     ys = []
-    for step in range(h.shape[0]):
+    for step in range(pz.shape[0]):
         S = (1.0 - z[step]) * S + z[step] * cand[step]
         ys.append(S * gate[step])
-    return matmul(torch.stack(ys), t[p + "o"], rounding)
+    return torch.stack(ys), S
+
+
+def mingru(h, t, p, rounding=None):
+    """``S_t = (1 - z_t) S_(t-1) + z_t c_t`` from a zero state; ``c = u + 1/2`` where ``u >= 0``,
+    ``sigmoid(u)`` below; the output is ``W_o (S_t * silu(W_g h))``."""
+    ys, _ = mingru_recurrence(matmul(h, t[p + "z"], rounding) + t[p + "z.b"].to(F64),
+                              matmul(h, t[p + "x"], rounding) + t[p + "x.b"].to(F64),
+                              matmul(h, t[p + "g"], rounding))
+    return matmul(ys, t[p + "o"], rounding)
 
 
 def dense_ff(h, t, p, rounding=None):
@@ -167,3 +176,17 @@ def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens: List[int], r
             layers_out.append(x.clone())
     x = group_rms_norm(x, t["final.norm"], groups, eps)
     return matmul(x, t["embed"], rounding)
+
+
+def read_model_dir(model_dir):
+    """(config.json as a dictionary, {tensor name: torch tensor}) of a model folder."""
+    import json
+    from pathlib import Path
+
+    from kappai_amd.weights.safetensors_io import SafetensorsFile
+    cfg = json.loads((Path(model_dir) / "config.json").read_text())
+    f = SafetensorsFile(Path(model_dir) / "model.safetensors")
+    try:
+        return cfg, {n: f.read(n) for n in f.names()}
+    finally:
+        f.close()
