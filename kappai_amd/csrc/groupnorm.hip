@@ -144,22 +144,24 @@ extern "C" int kappai_canon_conv(const float* h, const float* taps, float* state
 template <typename TT>
 __global__ __launch_bounds__(GN_THREADS) void scale_add_positions_kernel(
     float* __restrict__ x, float scale, const TT* __restrict__ table, const int* __restrict__ row_pos,
-    int D) {
+    int D, int n_positions) {
   const int t = blockIdx.x;
-  const TT* p = table + (size_t)row_pos[t] * D;
+  // (the host refuses a step past the table; a row of a warm-up run may carry any position)
+  const TT* p = table + (size_t)min(max(row_pos[t], 0), n_positions - 1) * D;
   for (int i = threadIdx.x; i < D; i += GN_THREADS)
     x[(size_t)t * D + i] = fmaf(x[(size_t)t * D + i], scale, to_f32(p[i]));
 }
 
 extern "C" int kappai_scale_add_positions(float* x, float scale, const void* table,
                                           int table_is_bf16, const int* row_pos, int T, int D,
-                                          hipStream_t stream) {
+                                          int n_positions, hipStream_t stream) {
   if (T <= 0) return 0;
+  if (n_positions < 1) return (int)hipErrorInvalidValue;
   if (table_is_bf16)
     hipLaunchKernelGGL(scale_add_positions_kernel<bf16_t>, dim3(T), dim3(GN_THREADS), 0, stream, x,
-                       scale, (const bf16_t*)table, row_pos, D);
+                       scale, (const bf16_t*)table, row_pos, D, n_positions);
   else
     hipLaunchKernelGGL(scale_add_positions_kernel<float>, dim3(T), dim3(GN_THREADS), 0, stream, x,
-                       scale, (const float*)table, row_pos, D);
+                       scale, (const float*)table, row_pos, D, n_positions);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }

@@ -233,6 +233,8 @@ class StepRunner:
         # what the model's parts want laid out beside the step's own tables
         tables = getattr(model, "step_tables", None)
         self.step_tables = list(tables()) if callable(tables) else []
+        limit = getattr(model, "position_limit", None)
+        self.position_limit = limit() if callable(limit) else None
 
     # -- the forward pass of a step ----------------------------------------------------------
     def forward(self, batch: RowBatch, workspace: Optional[Workspace] = None) -> torch.Tensor:
@@ -431,6 +433,13 @@ class StepRunner:
         if not entries:
             raise ValueError("a step needs at least one entry")
         single = all(len(e.tokens) == 1 for e in entries) and placed is None
+        if self.position_limit is not None:
+            for e in entries:
+                if e.cache.length + len(e.tokens) > self.position_limit:
+                    raise ValueError(
+                        f"request {e.cache.request_id!r} would reach position "
+                        f"{e.cache.length + len(e.tokens) - 1}; the model has rows for "
+                        f"{self.position_limit} positions")
         extended: List[StepEntry] = []
         try:
             for e in entries:

@@ -1226,7 +1226,8 @@ def canon_conv(h: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, row_pos
 
 def scale_add_positions(x: torch.Tensor, scale: float, table: torch.Tensor,
                         row_pos: torch.Tensor) -> None:
-    """``x[t] = x[t] * scale + table[row_pos[t]]`` in place on float32 rows."""
+    """``x[t] = x[t] * scale + table[row_pos[t]]`` in place on float32 rows.  The caller keeps
+    positions inside the table; the kernel reads no row outside it whatever ``row_pos`` holds."""
     _gpu("x", x, F32)
     _gpu("table", table, (F32, BF16))
     _gpu("row_pos", row_pos, I32)
@@ -1235,7 +1236,7 @@ def scale_add_positions(x: torch.Tensor, scale: float, table: torch.Tensor,
           lambda: f"scale_add_positions: x {tuple(x.shape)}, table {tuple(table.shape)}")
     check(library("groupnorm").kappai_scale_add_positions(
         _ptr(x), _c_float(scale), _ptr(table), _c_int(_is_bf16(table.dtype)), _ptr(row_pos),
-        _c_int(T), _c_int(D), _stream()), "scale_add_positions")
+        _c_int(T), _c_int(D), _c_int(table.shape[0]), _stream()), "scale_add_positions")
 
 
 GLU_SILU, GLU_GELU_TANH = 0, 1

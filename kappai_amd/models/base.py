@@ -116,6 +116,11 @@ class Model:
     def vocab_size(self) -> int:
         return self.config.vocab_size
 
+    def position_limit(self) -> Optional[int]:
+        """How many positions a sequence may have when positions enter through a table with a
+        row each (``embedding_position.max_positions``); None when nothing bounds them."""
+        return getattr(self.embedding_position, "max_positions", None)
+
     def first_norm(self):
         """What the last block of the schedule sees in place of a next block: the final norm and
         the head that takes its rows."""

@@ -14,7 +14,9 @@ class LearnedPositions(PositionEncoding):
     """``x[t] = x[t] * input_scale + table[position of t]``: the table's row is added as it is;
     ``input_scale`` is what the embedded rows are multiplied by first (an embedding's scale), so
     that scale and sum are one pass over the rows.  Positions count from 0 in every request and
-    must stay below ``max_positions``."""
+    must stay below ``max_positions``: the step function refuses a step that would go past
+    (``Model.position_limit``); a batch's ``max_position`` may be a bound only (a captured decode
+    graph's), so it is no test here."""
 
     def __init__(self, name: str, max_positions: int, width: int, input_scale: float = 1.0):
         self.name, self.max_positions, self.width = name, int(max_positions), width
@@ -28,9 +30,6 @@ class LearnedPositions(PositionEncoding):
         self.table = tensors[self.name].contiguous()
 
     def on_embedding(self, x: torch.Tensor, batch) -> None:
-        if batch.max_position >= self.max_positions:
-            raise ValueError(f"position {batch.max_position} is beyond the {self.max_positions} "
-                             f"positions that {self.name!r} has rows for")
         with profile.scope("embd"):
             ops.scale_add_positions(x, self.input_scale, self.table, batch.row_pos)
 

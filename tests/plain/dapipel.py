@@ -125,11 +125,16 @@ def dense_ff(h, t, p, rounding=None):
     return matmul(a, t[p + "down"], rounding)
 
 
-def moe_ff(h, t, p, experts: int, top: int, rounding=None):
+def moe_ff(h, t, p, experts: int, top: int, rounding=None, margins: Optional[list] = None):
     """Router logits over all experts, the ``top`` largest chosen, their weights the softmax over
-    the chosen logits alone; every expert is a SiLU-gated feed-forward."""
+    the chosen logits alone; every expert is a SiLU-gated feed-forward.  ``margins`` gets, per
+    row, how far the last chosen logit lies above the first one left out, relative to the row's
+    largest |logit| (a small margin is a close call that rounding may decide otherwise)."""
     logits = _r(h, rounding) @ t[p + "router"].to(F64).T
     best, chosen = torch.topk(logits, top, dim=-1)
+    if margins is not None and top < experts:
+        ranked = torch.sort(logits, dim=-1, descending=True).values
+        margins.append((ranked[:, top - 1] - ranked[:, top]) / logits.abs().max(dim=-1).values)
     weights = torch.softmax(best, dim=-1)
     out = torch.zeros(h.shape[0], t[p + "e0.down"].shape[0], dtype=F64)
     for e in range(experts):
@@ -145,9 +150,10 @@ def moe_ff(h, t, p, experts: int, top: int, rounding=None):
 
 
 def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens: List[int], rounding=None,
-            layers_out: Optional[list] = None) -> torch.Tensor:
+            layers_out: Optional[list] = None, margins: Optional[list] = None) -> torch.Tensor:
     """float64 logits [len(tokens), vocab] of one sequence from position 0.  ``layers_out``: a
-    list that gets the residual stream after every layer."""
+    list that gets the residual stream after every layer; ``margins``: one that gets every
+    router's margins (see ``moe_ff``)."""
     t = tensors
     eps, groups = config["norm"]["eps"], config["norm"]["groups"]
     ids = torch.tensor(tokens, dtype=torch.long)
@@ -169,7 +175,7 @@ def forward(config: dict, tensors: Dict[str, torch.Tensor], tokens: List[int], r
                 x = x + dense_ff(h, t, p + "mlp.", rounding)
             elif mlp["kind"] == "moe":
                 x = x + moe_ff(h, t, p + "mlp.", mlp["router"]["experts"], mlp["router"]["top"],
-                               rounding)
+                               rounding, margins)
             else:
                 raise ValueError(f"layer {li}: unknown feed-forward {mlp['kind']!r}")
         if layers_out is not None:

@@ -39,7 +39,7 @@ def test_config_reads_every_size_from_the_file():
     assert cfg.layers[1].mixer == {"heads": 4, "kv_heads": 2, "dim": 16, "vdim": 24, "scale": 0.3,
                                    "diff": 0.4, "window": 20}
     assert cfg.layers[2].mixer["window"] is None and cfg.layers[2].mlp is None
-    assert cfg.layers[0].mlp == {"kind": "moe", "ff": 40, "experts": 6, "top": 3}
+    assert cfg.layers[0].mlp == {"kind": "moe", "ff": 40, "experts": 5, "top": 2}
     assert cfg.to_dict() == raw
 
 
@@ -48,7 +48,7 @@ def test_config_reads_every_size_from_the_file():
     (lambda c: c["norm"].update(groups=5), "groups"),
     (lambda c: c["layers"][1].update(type="conv"), "type"),
     (lambda c: c["layers"][1]["mixer"].update(kv_heads=3), "kv heads"),
-    (lambda c: c["layers"][0]["mlp"]["router"].update(top=7), "top"),
+    (lambda c: c["layers"][0]["mlp"]["router"].update(top=6), "top"),
     (lambda c: c["layers"][3]["mlp"].update(kind="sparse"), "kind"),
     (lambda c: c["layers"][1]["mixer"].pop("scale"), "scale"),
     (lambda c: c.update(canon=None), "canon"),
@@ -68,7 +68,7 @@ def test_tensor_names_and_shapes():
     assert shapes["l0.mix.z"] == (80, 96) and shapes["l0.mix.z.b"] == (80,)
     assert shapes["l0.mix.x.b"] == (80,) and "l0.mix.g.b" not in shapes
     assert shapes["l0.mix.o"] == (96, 80)
-    assert shapes["l0.mlp.router"] == (6, 96) and shapes["l0.mlp.e5.down"] == (96, 40)
+    assert shapes["l0.mlp.router"] == (5, 96) and shapes["l0.mlp.e4.down"] == (96, 40)
     assert shapes["l1.mix.q"] == (4 * 2 * 16, 96) and shapes["l1.mix.k"] == (2 * 2 * 16, 96)
     assert shapes["l1.mix.v"] == (2 * 24, 96) and shapes["l1.mix.o"] == (96, 4 * 24)
     assert shapes["l1.mix.lq1"] == (16,) and shapes["l1.canon2"] == (96, 3)
