@@ -101,6 +101,104 @@ def run_workload(key, dtype, device, repeat_penalty=1.0):
     return 0
 
 
+# --compare: the Dapipel decoder beside the LFM2 shape of the same width, depth, attention layers
+# and feed-forward width (config/shapes.py), both with random weights
+COMPARISONS = {"w1024": ("dapipel-w1024", "lfm2-like-w1024"),
+               "w2048": ("dapipel-w2048", "lfm2-like-w2048")}
+
+
+def stage_table(runner, entries_of, reps):
+    """{stage: microseconds a step} of ``reps`` steps run part by part with events around every
+    stage (``entries_of(i)`` gives step i's entries)."""
+    from kappai_amd.kernels import profile
+    graphs, runner.decode_graphs = runner.decode_graphs, False
+    profile.STAGE_TIMES.start()
+    try:
+        for i in range(reps):
+            runner.step(entries_of(i))
+        tot = profile.STAGE_TIMES.totals()
+    finally:
+        profile.STAGE_TIMES.stop()
+        profile.STAGE_TIMES.reset()
+        runner.decode_graphs = graphs
+    return {k: round(v[0] / reps, 1) for k, v in sorted(tot.items())}
+
+
+def measure_model(name, dtype, device, prefill_tokens, batch, context, steps, warmup, page_size):
+    """Prompt steps of ``prefill_tokens`` tokens and decode steps of ``batch`` requests at
+    ``context`` tokens for the named shape: tokens a second, and the time of a step by stage."""
+    import torch
+
+    from kappai_amd.cache import CacheManager
+    from kappai_amd.engine import StepEntry, StepRunner
+    model = random_model(_shape(name), dtype, device)
+    out = {"model": name, "weight_mb_a_step": round(model.weight_bytes_per_step() / 1e6, 1)}
+    # prompt steps: requests of one portion each, queued one behind the other
+    pages = (prefill_tokens + page_size - 1) // page_size
+    cache = CacheManager(model.cache_specs(), page_size, pages, 1)
+    cache.allocate_storage(model.dtype, device)
+    runner = StepRunner(model, cache, device)
+    gen = torch.Generator().manual_seed(7)
+    prompt = torch.randint(0, model.vocab_size, (prefill_tokens,), generator=gen).tolist()
+
+    def one_prompt(_=0):
+        rc = cache.open("p")
+        runner.step([StepEntry(rc, prompt, [prefill_tokens - 1])])
+        cache.close(rc)
+
+    for _ in range(3):
+        one_prompt()
+    sync()
+    reps = 8
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        one_prompt()
+    sync()
+    dt = (time.perf_counter() - t0) / reps
+    out["prefill_ms"] = round(dt * 1e3, 3)
+    out["prefill_tok_s"] = round(prefill_tokens / dt, 1)
+    live = {}
+
+    def prompt_entries(i):
+        if "rc" in live:
+            cache.close(live.pop("rc"))
+        live["rc"] = cache.open(("t", i))
+        return [StepEntry(live["rc"], prompt, [prefill_tokens - 1])]
+
+    out["prefill_stages_us"] = stage_table(runner, prompt_entries, 3)
+    if "rc" in live:
+        cache.close(live.pop("rc"))
+    del runner, cache
+    torch.cuda.empty_cache()
+    # decode steps
+    b = DecodeBench(model, batch, context - (steps + warmup) - 8, context, page_size, device)
+    dt = b.run(warmup, steps)
+    out["decode_ms"] = round(dt / steps * 1e3, 4)
+    out["decode_tok_s"] = round(batch * steps / dt, 1)
+    out["decode_stages_us"] = stage_table(
+        b.runner, lambda i: [StepEntry(rc, [1], [0]) for rc in b.requests], 4)
+    b.close()
+    del b, model
+    torch.cuda.empty_cache()
+    return out
+
+
+def run_comparison(keys, args):
+    results = {}
+    for key in keys:
+        new, old = COMPARISONS[key]
+        results[key] = [measure_model(n, args.dtype, "cuda:0", args.prefill_tokens, args.batch,
+                                      min(args.context, 2048), args.steps, args.warmup,
+                                      args.page_size) for n in (new, old)]
+        print(f"bench.py: {key} done", file=sys.stderr, flush=True)
+    print(json.dumps({"metric": "prefill and decode tok/s, Dapipel beside the LFM2 shape of equal "
+                                "size", "unit": "tok/s", "n_gpus": 1, "dtype": args.dtype,
+                      "data": "synthetic", "prefill_tokens": args.prefill_tokens,
+                      "batch": args.batch, "context": min(args.context, 2048),
+                      "steps": args.steps, "warmup": args.warmup, "sizes": results}))
+    return 0
+
+
 def random_model(raw, dtype, device, seed=0, std=0.02):
     """The model of ``raw`` with N(0, std) weights (norm weights 1), through the framework's own
     random-weights mode and loader: the folder is written once (under the temp folder, named by
@@ -464,7 +562,21 @@ def main() -> int:
     ap.add_argument("--repeat-penalty", type=float, default=1.0,
                     help="serving workloads: a repeat penalty over the last 64 tokens before "
                          "the greedy choice (1: none)")
+    ap.add_argument("--compare", default="", metavar="SIZES",
+                    help="instead of the headline run: prompt and decode steps of the Dapipel "
+                         "decoder beside the LFM2 shape of equal size, at these sizes (comma "
+                         "separated: " + ", ".join(sorted(COMPARISONS)) + "; 'all')")
     args = ap.parse_args()
+    if args.compare:
+        keys = sorted(COMPARISONS) if args.compare == "all" else args.compare.split(",")
+        for k in keys:
+            if k not in COMPARISONS:
+                print(f"bench.py: no comparison {k!r}; known: {', '.join(sorted(COMPARISONS))}")
+                return 2
+        if args.gpus != 1:
+            print("bench.py: this engine runs on one GPU; --gpus must be 1")
+            return 2
+        return run_comparison(keys, args)
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus must be 1 (nothing was measured)")
         return 2

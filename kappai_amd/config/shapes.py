@@ -59,6 +59,47 @@ SHAPES: Dict[str, dict] = {
 }
 
 
+def _dapipel(width, mixers, heads, kv_heads, dim, vdim, window, ff, experts, top, vocab=65536,
+             positions=8192, inner=None) -> dict:
+    """Layers by letter: "a" windowed differential attention, "g" minGRU; dense feed-forwards of
+    ``ff`` and mixtures of ``experts`` experts of ``ff * 2 // (top * 2)`` (as many active weights
+    as the dense layer) in turns."""
+    layers = []
+    for i, kind in enumerate(mixers):
+        if kind == "a":
+            mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim,
+                     "scale": dim ** -0.5, "diff": 0.8, "mask": {"size": window}}
+        else:
+            mixer = {"width": inner or width}
+        mlp = ({"kind": "dense", "ff": ff} if i % 2 == 0 else
+               {"kind": "moe", "expert": {"ff": ff // top}, "router": {"experts": experts,
+                                                                       "top": top}})
+        layers.append({"type": "attention" if kind == "a" else "mingru", "mixer": mixer,
+                       "mlp": mlp})
+    return {"architecture": "Dapipel", "vocab": vocab, "width": width, "max_positions": positions,
+            "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5, "groups": 8},
+            "canon": {"taps": 4}, "layers": layers}
+
+
+SHAPES.update({
+    # eight layers at a width of 1024: attention where the LFM2 pattern has it (2, 5, 7), a
+    # recurrent layer elsewhere; feed-forward 4608 dense or 16 experts of 2304, two a token
+    "dapipel-w1024": _dapipel(1024, "ggaggaga", 16, 8, 32, 64, 1024, 4608, 16, 2),
+    # the same at a width of 2048: heads of 128 values on maps of 64, feed-forward 8192
+    "dapipel-w2048": _dapipel(2048, "ggaggaga", 16, 8, 64, 128, 2048, 8192, 16, 2),
+    # a tiny one for smoke runs
+    "dapipel-tiny": _dapipel(64, "gaga", 4, 2, 8, 16, 24, 96, 4, 2, vocab=256, positions=512,
+                             inner=48),
+})
+# the LFM2 shapes of the same widths, depths, attention layers and feed-forward widths
+SHAPES.update({
+    "lfm2-like-w1024": _lfm2(1024, 8, (2, 5, 7), 16, 8, 4608, block_auto_adjust_ff_dim=False,
+                             max_position_embeddings=8192),
+    "lfm2-like-w2048": _lfm2(2048, 8, (2, 5, 7), 32, 8, 8192, block_auto_adjust_ff_dim=False,
+                             max_position_embeddings=8192),
+})
+
+
 def named_shape(name: str) -> dict:
     """A copy of the configuration called ``name`` (any case), or a ``KeyError`` naming them all."""
     key = name.strip().lower()

@@ -140,6 +140,92 @@ extern "C" int kappai_canon_conv(const float* h, const float* taps, float* state
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
+// A step of single rows (every segment one decoded token): residual sum, norm, convolution and
+// the state's shift in one kernel, a block a row.  Row t is segment t; its history is all state.
+template <typename TO>
+__global__ __launch_bounds__(GN_THREADS) void add_group_rmsnorm_canon_step_kernel(
+    float* __restrict__ resid, const void* __restrict__ delta, int delta_kind, int n_part,
+    size_t part_stride, const float* __restrict__ w, float eps, int groups, int D,
+    const float* __restrict__ taps, float* __restrict__ state, const int* __restrict__ row_pos,
+    const int* __restrict__ seg_slot, int n_taps, TO* __restrict__ out) {
+  extern __shared__ float row[];
+  float* scale = row + D;
+  const int r = blockIdx.x;
+  float* x = resid + (size_t)r * D;
+  for (int i = threadIdx.x; i < D; i += GN_THREADS) {
+    float v = x[i];
+    if (delta_kind == 1) {
+      v += bf16_to_f32(((const bf16_t*)delta)[(size_t)r * D + i]);
+    } else if (delta_kind == 2) {
+      const float* p = (const float*)delta + (size_t)r * D + i;
+      for (int s = 0; s < n_part; ++s) v += p[s * part_stride];
+    }
+    row[i] = v;
+    if (delta_kind) x[i] = v;
+  }
+  __syncthreads();
+  const int gs = D / groups;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  for (int g = wave; g < groups; g += GN_THREADS / WAVE) {
+    float ss = 0.f;
+    for (int i = lane; i < gs; i += WAVE) {
+      const float v = row[g * gs + i];
+      ss = fmaf(v, v, ss);
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) scale[g] = 1.0f / sqrtf(ss / (float)gs + eps);
+  }
+  __syncthreads();
+  const int pos = row_pos[r];
+  float* st = state + (size_t)seg_slot[r] * (n_taps - 1) * D;
+  for (int c = threadIdx.x; c < D; c += GN_THREADS) {
+    // state[k] is the input n - 1 - k places back; everything is asked for before it is used
+    float keep[CANON_MAX_TAPS], tw[CANON_MAX_TAPS];
+#pragma unroll
+    for (int k = 0; k < CANON_MAX_TAPS; ++k) {
+      if (k < n_taps) tw[k] = taps[(size_t)c * n_taps + k];
+      if (k < n_taps - 1) keep[k] = pos - (n_taps - 1 - k) >= 0 ? st[(size_t)k * D + c] : 0.f;
+    }
+    const float h = row[c] * scale[c / gs] * w[c];
+    float acc = h;
+#pragma unroll
+    for (int k = 0; k < CANON_MAX_TAPS; ++k) {
+      if (k < n_taps - 1) {
+        acc = fmaf(tw[k], keep[k], acc);
+        if (k > 0) st[(size_t)(k - 1) * D + c] = keep[k];      // one place older now
+      } else if (k == n_taps - 1) {
+        acc = fmaf(tw[k], h, acc);
+      }
+    }
+    if (n_taps > 1) st[(size_t)(n_taps - 2) * D + c] = h;
+    from_f32(out + (size_t)r * D + c, acc);
+  }
+}
+
+extern "C" int kappai_add_group_rmsnorm_canon_step(float* resid, const void* delta, int delta_kind,
+                                                   int n_part, int T, int D, const float* w,
+                                                   float eps, int groups, const float* taps,
+                                                   float* state, const int* row_pos,
+                                                   const int* seg_slot, int n_taps, void* out,
+                                                   int out_is_bf16, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (groups < 1 || D % groups || delta_kind < 0 || delta_kind > 2 || n_taps < 1 ||
+      n_taps > CANON_MAX_TAPS)
+    return (int)hipErrorInvalidValue;
+  const size_t lds = (size_t)(D + groups) * sizeof(float);
+  if (lds > 64 * 1024) return (int)hipErrorInvalidValue;
+  const size_t ps = (size_t)T * D;
+  if (out_is_bf16)
+    hipLaunchKernelGGL(add_group_rmsnorm_canon_step_kernel<bf16_t>, dim3(T), dim3(GN_THREADS), lds,
+                       stream, resid, delta, delta_kind, n_part, ps, w, eps, groups, D, taps, state,
+                       row_pos, seg_slot, n_taps, (bf16_t*)out);
+  else
+    hipLaunchKernelGGL(add_group_rmsnorm_canon_step_kernel<float>, dim3(T), dim3(GN_THREADS), lds,
+                       stream, resid, delta, delta_kind, n_part, ps, w, eps, groups, D, taps, state,
+                       row_pos, seg_slot, n_taps, (float*)out);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
 // x[t] = x[t] * scale + table[row_pos[t]]: the embedding's scale and a learned row per position.
 template <typename TT>
 __global__ __launch_bounds__(GN_THREADS) void scale_add_positions_kernel(

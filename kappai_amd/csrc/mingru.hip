@@ -1,11 +1,11 @@
 // minGRU: S_t = (1 - z_t) S_(t-1) + z_t c_t per channel, z = sigmoid(pz), c = pu + 1/2 where
 // pu >= 0 and sigmoid(pu) below, y_t = S_t * silu(pg).  The projections [T, 3W] = (pz | pu | pg)
-// come in float32 with their biases added; gates, candidates and the state are float32; the state
-// lives in a slot per request [slots, W] and a segment that starts at position 0 starts from zero.
+// come with their biases added, in float32 or as the bfloat16 a product stored; gates, candidates
+// and the state are float32; the state lives in a slot per request [slots, W] and a segment that
+// starts at position 0 starts from zero.
 #include "common.h"
 
 #define MG_THREADS 256
-#define MG_CHUNK 32          // rows a thread of the chunked scan walks
 
 __device__ __forceinline__ float sigmoid_f(float x) { return 1.0f / (1.0f + expf(-x)); }
 
@@ -18,9 +18,9 @@ __device__ __forceinline__ void mingru_gates(float pz, float pu, float& a, float
 
 // One thread a (segment, channel), walking the segment's rows in order: what a step of few rows
 // a request runs (decoding, short portions).
-template <typename TO>
+template <typename TP, typename TO>
 __global__ __launch_bounds__(MG_THREADS) void mingru_scan_rows_kernel(
-    const float* __restrict__ proj, float* __restrict__ state, const int* __restrict__ seg_start,
+    const TP* __restrict__ proj, float* __restrict__ state, const int* __restrict__ seg_start,
     const int* __restrict__ seg_pos0, const int* __restrict__ seg_slot, int W,
     TO* __restrict__ out) {
   const int seg = blockIdx.y;
@@ -30,11 +30,11 @@ __global__ __launch_bounds__(MG_THREADS) void mingru_scan_rows_kernel(
   float* st = state + (size_t)seg_slot[seg] * W + c;
   float S = seg_pos0[seg] > 0 ? *st : 0.f;
   for (int t = first; t < last; ++t) {
-    const float* p = proj + (size_t)t * 3 * W + c;
+    const TP* p = proj + (size_t)t * 3 * W + c;
     float a, b;
-    mingru_gates(p[0], p[W], a, b);
+    mingru_gates(to_f32(p[0]), to_f32(p[W]), a, b);
     S = fmaf(a, S, b);
-    const float g = p[2 * W];
+    const float g = to_f32(p[2 * W]);
     from_f32(out + (size_t)t * W + c, S * (g * sigmoid_f(g)));
   }
   *st = S;
@@ -42,28 +42,40 @@ __global__ __launch_bounds__(MG_THREADS) void mingru_scan_rows_kernel(
 
 // Long segments, three passes.  The recurrence S -> a S + b composes: a run of rows acts on the
 // state that enters it as S -> A S + B with A the product of its a and B its own result from
-// zero.  Pass 1: every chunk of MG_CHUNK rows of a segment gets its (A, B).  Pass 2: a thread a
+// zero.  Pass 1: every chunk of rows of a segment (the host cuts them) gets its (A, B).  Pass 2: a thread a
 // (segment, channel) carries the state over the chunks' (A, B) in order and leaves the state at
 // every chunk's start in place of them.  Pass 3: every chunk walks its rows from that state and
 // writes the outputs.  The state a row sees is the same sum of products whatever the chunks are,
 // up to rounding.
+template <typename TP>
 __global__ __launch_bounds__(MG_THREADS) void mingru_chunk_sums_kernel(
-    const float* __restrict__ proj, const int* __restrict__ chunks, int W,
+    const TP* __restrict__ proj, const int* __restrict__ chunks, int W,
     float* __restrict__ carry) {
   const int ch = blockIdx.y;
   const int c = blockIdx.x * MG_THREADS + threadIdx.x;
   if (c >= W) return;
   const int first = chunks[3 * ch + 1], n = chunks[3 * ch + 2];
   float A = 1.f, B = 0.f;
-  for (int t = first; t < first + n; ++t) {
-    const float* p = proj + (size_t)t * 3 * W + c;
-    float a, b;
-    mingru_gates(p[0], p[W], a, b);
-    A *= a;
-    B = fmaf(a, B, b);
+  // (four rows' loads at a time, so that they do not wait for one another)
+  for (int t0 = first; t0 < first + n; t0 += 4) {
+    float pz[4], pu[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const TP* p = proj + (size_t)min(t0 + i, first + n - 1) * 3 * W + c;
+      pz[i] = to_f32(p[0]);
+      pu[i] = to_f32(p[W]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (t0 + i >= first + n) break;
+      float a, b;
+      mingru_gates(pz[i], pu[i], a, b);
+      A *= a;
+      B = fmaf(a, B, b);
+    }
   }
-  carry[((size_t)ch * 2) * W + c] = A;
-  carry[((size_t)ch * 2 + 1) * W + c] = B;
+  carry[((size_t)ch * 3) * W + c] = A;
+  carry[((size_t)ch * 3 + 1) * W + c] = B;
 }
 
 __global__ __launch_bounds__(MG_THREADS) void mingru_chunk_carry_kernel(
@@ -75,64 +87,97 @@ __global__ __launch_bounds__(MG_THREADS) void mingru_chunk_carry_kernel(
   if (c >= W) return;
   float* st = state + (size_t)seg_slot[seg] * W + c;
   float S = seg_pos0[seg] > 0 ? *st : 0.f;
-  for (int ch = seg_chunk0[seg]; ch < seg_chunk0[seg + 1]; ++ch) {
-    const float A = carry[((size_t)ch * 2) * W + c], B = carry[((size_t)ch * 2 + 1) * W + c];
-    carry[((size_t)ch * 2) * W + c] = S;
-    S = fmaf(A, S, B);
+  const int ch1 = seg_chunk0[seg + 1];
+  for (int ch0 = seg_chunk0[seg]; ch0 < ch1; ch0 += 8) {
+    float A[8], B[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const size_t ch = (size_t)min(ch0 + i, ch1 - 1);
+      A[i] = carry[(ch * 3) * W + c];
+      B[i] = carry[(ch * 3 + 1) * W + c];
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      if (ch0 + i >= ch1) break;
+      carry[((size_t)(ch0 + i) * 3 + 2) * W + c] = S;      // the state the chunk starts from
+      S = fmaf(A[i], S, B[i]);
+    }
   }
   *st = S;
 }
 
-template <typename TO>
+template <typename TP, typename TO>
 __global__ __launch_bounds__(MG_THREADS) void mingru_chunk_out_kernel(
-    const float* __restrict__ proj, const int* __restrict__ chunks, int W,
+    const TP* __restrict__ proj, const int* __restrict__ chunks, int W,
     const float* __restrict__ carry, TO* __restrict__ out) {
   const int ch = blockIdx.y;
   const int c = blockIdx.x * MG_THREADS + threadIdx.x;
   if (c >= W) return;
   const int first = chunks[3 * ch + 1], n = chunks[3 * ch + 2];
-  float S = carry[((size_t)ch * 2) * W + c];
-  for (int t = first; t < first + n; ++t) {
-    const float* p = proj + (size_t)t * 3 * W + c;
-    float a, b;
-    mingru_gates(p[0], p[W], a, b);
-    S = fmaf(a, S, b);
-    const float g = p[2 * W];
-    from_f32(out + (size_t)t * W + c, S * (g * sigmoid_f(g)));
+  float S = carry[((size_t)ch * 3 + 2) * W + c];
+  for (int t0 = first; t0 < first + n; t0 += 4) {
+    float pz[4], pu[4], pg[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const TP* p = proj + (size_t)min(t0 + i, first + n - 1) * 3 * W + c;
+      pz[i] = to_f32(p[0]);
+      pu[i] = to_f32(p[W]);
+      pg[i] = to_f32(p[2 * W]);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      if (t0 + i >= first + n) break;
+      float a, b;
+      mingru_gates(pz[i], pu[i], a, b);
+      S = fmaf(a, S, b);
+      from_f32(out + (size_t)(t0 + i) * W + c, S * (pg[i] * sigmoid_f(pg[i])));
+    }
   }
 }
 
-extern "C" int kappai_mingru_chunk_rows() { return MG_CHUNK; }
-
-// `chunks` [n_chunks, 3] = (segment, first row, rows) and `seg_chunk0` [S + 1] (first chunk of
-// every segment) choose the three-pass form, with `carry` [n_chunks, 2, W] floats of scratch;
-// without them every segment is walked by one thread a channel.
-extern "C" int kappai_mingru_scan(const float* proj, float* state, const int* seg_start,
-                                  const int* seg_pos0, const int* seg_slot, int T, int S, int W,
-                                  const int* chunks, const int* seg_chunk0, int n_chunks,
-                                  float* carry, void* out, int out_is_bf16, hipStream_t stream) {
-  if (T <= 0 || S <= 0) return 0;
-  if (S > 65535 || n_chunks > 65535) return (int)hipErrorInvalidValue;
+template <typename TP, typename TO>
+static void mingru_launch(const void* proj_v, float* state, const int* seg_start,
+                          const int* seg_pos0, const int* seg_slot, int S, int W, const int* chunks,
+                          const int* seg_chunk0, int n_chunks, float* carry, void* out_v,
+                          hipStream_t stream) {
+  const TP* proj = (const TP*)proj_v;
+  TO* out = (TO*)out_v;
   const int bx = (W + MG_THREADS - 1) / MG_THREADS;
   if (chunks == nullptr) {
-    if (out_is_bf16)
-      hipLaunchKernelGGL(mingru_scan_rows_kernel<bf16_t>, dim3(bx, S), dim3(MG_THREADS), 0, stream,
-                         proj, state, seg_start, seg_pos0, seg_slot, W, (bf16_t*)out);
-    else
-      hipLaunchKernelGGL(mingru_scan_rows_kernel<float>, dim3(bx, S), dim3(MG_THREADS), 0, stream,
-                         proj, state, seg_start, seg_pos0, seg_slot, W, (float*)out);
-    KAPPAI_RETURN_LAUNCH_STATUS();
+    hipLaunchKernelGGL((mingru_scan_rows_kernel<TP, TO>), dim3(bx, S), dim3(MG_THREADS), 0, stream,
+                       proj, state, seg_start, seg_pos0, seg_slot, W, out);
+    return;
   }
-  if (n_chunks <= 0 || carry == nullptr || seg_chunk0 == nullptr) return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(mingru_chunk_sums_kernel, dim3(bx, n_chunks), dim3(MG_THREADS), 0, stream,
+  hipLaunchKernelGGL(mingru_chunk_sums_kernel<TP>, dim3(bx, n_chunks), dim3(MG_THREADS), 0, stream,
                      proj, chunks, W, carry);
   hipLaunchKernelGGL(mingru_chunk_carry_kernel, dim3(bx, S), dim3(MG_THREADS), 0, stream,
                      seg_chunk0, seg_pos0, seg_slot, W, carry, state);
-  if (out_is_bf16)
-    hipLaunchKernelGGL(mingru_chunk_out_kernel<bf16_t>, dim3(bx, n_chunks), dim3(MG_THREADS), 0,
-                       stream, proj, chunks, W, carry, (bf16_t*)out);
+  hipLaunchKernelGGL((mingru_chunk_out_kernel<TP, TO>), dim3(bx, n_chunks), dim3(MG_THREADS), 0,
+                     stream, proj, chunks, W, carry, out);
+}
+
+// `chunks` [n_chunks, 3] = (segment, first row, rows) and `seg_chunk0` [S + 1] (first chunk of
+// every segment) choose the three-pass form, with `carry` [n_chunks, 3, W] floats of scratch
+// (a chunk's A and B, and the state it starts from);
+// without them every segment is walked by one thread a channel.
+extern "C" int kappai_mingru_scan(const void* proj, int proj_is_bf16, float* state,
+                                  const int* seg_start, const int* seg_pos0, const int* seg_slot,
+                                  int T, int S, int W, const int* chunks, const int* seg_chunk0,
+                                  int n_chunks, float* carry, void* out, int out_is_bf16,
+                                  hipStream_t stream) {
+  if (T <= 0 || S <= 0) return 0;
+  if (S > 65535 || n_chunks > 65535) return (int)hipErrorInvalidValue;
+  if (chunks != nullptr && (n_chunks <= 0 || carry == nullptr || seg_chunk0 == nullptr))
+    return (int)hipErrorInvalidValue;
+  if (proj_is_bf16 && !out_is_bf16) return (int)hipErrorInvalidValue;
+  if (proj_is_bf16)
+    mingru_launch<bf16_t, bf16_t>(proj, state, seg_start, seg_pos0, seg_slot, S, W, chunks,
+                                  seg_chunk0, n_chunks, carry, out, stream);
+  else if (out_is_bf16)
+    mingru_launch<float, bf16_t>(proj, state, seg_start, seg_pos0, seg_slot, S, W, chunks,
+                                 seg_chunk0, n_chunks, carry, out, stream);
   else
-    hipLaunchKernelGGL(mingru_chunk_out_kernel<float>, dim3(bx, n_chunks), dim3(MG_THREADS), 0,
-                       stream, proj, chunks, W, carry, (float*)out);
+    mingru_launch<float, float>(proj, state, seg_start, seg_pos0, seg_slot, S, W, chunks,
+                                seg_chunk0, n_chunks, carry, out, stream);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }

@@ -9,13 +9,16 @@
 //   moe_combine   out[t] = sum_k weight[t, k] * y[slot of (t, k)], in the order of k, float32
 #include "common.h"
 
-#define MOE_TILE_M 32
+#define MOE_TILE_M 64          // slots of a tile (the matrix-core kernel: four row tiles of 16)
+#define MOE_HALF_M 32          // rows a block of the plain kernel takes: half a tile
 #define MOE_TILE_N 64
 #define MOE_TILE_K 32
 #define MOE_MAX_TOP 16
 #define MOE_THREADS 256
 
 extern "C" int kappai_moe_tile_rows() { return MOE_TILE_M; }
+
+#define MOE_ROUTE_GROUP 8       // experts whose sums a lane carries side by side
 
 template <typename T>
 __global__ __launch_bounds__(MOE_THREADS) void moe_route_kernel(
@@ -27,12 +30,26 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_route_kernel(
   const int row = row_raw < n_rows ? row_raw : n_rows - 1;
   float* logits = logits_all + wave * E;
   const T* xr = x + (size_t)row * ldx;
-  for (int e = 0; e < E; ++e) {
-    const float* r = router + (size_t)e * D;
-    float acc = 0.f;
-    for (int c = lane; c < D; c += WAVE) acc = fmaf(to_f32(xr[c]), r[c], acc);
-    acc = wave_sum(acc);
-    if (lane == 0) logits[e] = acc;
+  // a wave a row; the lanes stride over the row, each with the sums of a group of experts, so
+  // that the loads of a pass do not wait for one another
+  for (int e0 = 0; e0 < E; e0 += MOE_ROUTE_GROUP) {
+    float acc[MOE_ROUTE_GROUP];
+#pragma unroll
+    for (int j = 0; j < MOE_ROUTE_GROUP; ++j) acc[j] = 0.f;
+#pragma unroll 4
+    for (int c = lane; c < D; c += WAVE) {
+      const float xv = to_f32(xr[c]);
+#pragma unroll
+      for (int j = 0; j < MOE_ROUTE_GROUP; ++j) {
+        const int e = min(e0 + j, E - 1);
+        acc[j] = fmaf(xv, router[(size_t)e * D + c], acc[j]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < MOE_ROUTE_GROUP; ++j) {
+      const float sum = wave_sum(acc[j]);
+      if (lane == 0 && e0 + j < E) logits[e0 + j] = sum;
+    }
   }
   __syncthreads();
   float cv[MOE_MAX_TOP];
@@ -85,58 +102,90 @@ extern "C" int kappai_moe_route(const void* x, int ldx, int x_is_bf16, const flo
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
-// One wave sorts the pairs by expert, stably: 64 pairs at a time, the lanes with the same expert
-// found by ballots, their places by counting the lanes below.  Pass 1 counts, pass 2 places.
-__global__ __launch_bounds__(WAVE) void moe_plan_kernel(
-    const int* __restrict__ idx, int P, int E, int n_tiles, int* __restrict__ slot_of_pair,
-    int* __restrict__ pair_of_slot, int* __restrict__ tile_expert) {
-  extern __shared__ int plan_lds[];
-  int* count = plan_lds;           // pairs of the expert; in pass 2: pairs placed so far
-  int* base = plan_lds + E;        // first slot of the expert
-  const int lane = threadIdx.x;
-  for (int e = lane; e < E; e += WAVE) count[e] = 0;
-  for (int i = lane; i < n_tiles * MOE_TILE_M; i += WAVE) pair_of_slot[i] = -1;
-  for (int i = lane; i < n_tiles; i += WAVE) tile_expert[i] = -1;
-  __syncthreads();
-  for (int pass = 0; pass < 2; ++pass) {
-    for (int p0 = 0; p0 < P; p0 += WAVE) {
-      const int p = p0 + lane;
-      const int e = p < P ? idx[p] : -1;
-      bool todo = p < P;
-      while (true) {
-        const unsigned long long rest = __ballot(todo);
-        if (!rest) break;
-        const int leader = __ffsll((long long)rest) - 1;
-        const int cur = __shfl(e, leader);
-        const bool mine = todo && e == cur;
-        const unsigned long long mask = __ballot(mine);
-        const int before = count[cur];
-        __syncthreads();
-        if (pass == 1 && mine) {
-          const int rank = __popcll(mask & ((1ull << lane) - 1ull));
-          const int slot = base[cur] + before + rank;
-          slot_of_pair[p] = slot;
-          pair_of_slot[slot] = p;
-        }
-        if (lane == 0) count[cur] = before + __popcll(mask);
-        __syncthreads();
-        if (mine) todo = false;
+// The pairs sorted by expert, stably and without atomics.  The waves of one block each take a
+// run of the pairs, 64 at a time: the lanes with the same expert are found by ballots and placed
+// by counting the lanes below.  Pass 1 counts per wave and expert; then every expert's run gets
+// its first slot (a multiple of MOE_TILE_M) and every wave its place in the run; pass 2 places.
+#define MOE_PLAN_MAX_WAVES 16
+
+__device__ __forceinline__ void moe_plan_pass(const int* __restrict__ idx, int p_lo, int p_hi,
+                                              int* cnt, const int* start, bool place,
+                                              int* __restrict__ slot_of_pair,
+                                              int* __restrict__ pair_of_slot) {
+  const int lane = threadIdx.x % WAVE;
+  for (int p0 = p_lo; p0 < p_hi; p0 += WAVE) {
+    const int p = p0 + lane;
+    const int e = p < p_hi ? idx[p] : -1;
+    bool todo = p < p_hi;
+    while (true) {
+      const unsigned long long rest = __ballot(todo);
+      if (!rest) break;
+      const int cur = __shfl(e, __ffsll((long long)rest) - 1);
+      const bool mine = todo && e == cur;
+      const unsigned long long mask = __ballot(mine);
+      const int before = cnt[cur];          // (only this wave writes its counters)
+      if (place && mine) {
+        const int slot = start[cur] + before + __popcll(mask & ((1ull << lane) - 1ull));
+        slot_of_pair[p] = slot;
+        pair_of_slot[slot] = p;
       }
-    }
-    if (pass == 0) {
-      if (lane == 0) {
-        int at = 0;
-        for (int e = 0; e < E; ++e) {
-          base[e] = at;
-          const int tiles = (count[e] + MOE_TILE_M - 1) / MOE_TILE_M;
-          for (int i = 0; i < tiles; ++i) tile_expert[at / MOE_TILE_M + i] = e;
-          at += tiles * MOE_TILE_M;
-          count[e] = 0;
-        }
-      }
-      __syncthreads();
+      __builtin_amdgcn_wave_barrier();
+      if (lane == 0) cnt[cur] = before + __popcll(mask);
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
+      if (mine) todo = false;
     }
   }
+}
+
+__global__ __launch_bounds__(MOE_PLAN_MAX_WAVES * WAVE) void moe_plan_kernel(
+    const int* __restrict__ idx, int P, int E, int n_tiles, int n_waves,
+    int* __restrict__ slot_of_pair, int* __restrict__ pair_of_slot,
+    int* __restrict__ tile_expert) {
+  extern __shared__ int plan_lds[];
+  int* base = plan_lds;                 // [E] first slot of the expert's run
+  int* len = plan_lds + E;              // [E] pairs of the expert
+  int* cnt = plan_lds + 2 * E;          // [n_waves][E] pairs of the wave; then placed so far
+  int* start = cnt + n_waves * E;       // [n_waves][E] first slot of the wave's pairs of e
+  const int tid = threadIdx.x, nt = blockDim.x;
+  const int wave = tid / WAVE;
+  for (int i = tid; i < n_waves * E; i += nt) cnt[i] = 0;
+  for (int i = tid; i < n_tiles * MOE_TILE_M; i += nt) pair_of_slot[i] = -1;
+  for (int i = tid; i < n_tiles; i += nt) tile_expert[i] = -1;
+  __syncthreads();
+  const int per = ((P + n_waves * WAVE - 1) / (n_waves * WAVE)) * WAVE;
+  const int p_lo = min(P, wave * per), p_hi = min(P, p_lo + per);
+  moe_plan_pass(idx, p_lo, p_hi, cnt + wave * E, nullptr, false, slot_of_pair, pair_of_slot);
+  __syncthreads();
+  // the runs' lengths and, inside a run, the waves one after the other
+  for (int e = tid; e < E; e += nt) {
+    int sum = 0;
+    for (int w = 0; w < n_waves; ++w) {
+      const int c = cnt[w * E + e];
+      start[w * E + e] = sum;
+      sum += c;
+      cnt[w * E + e] = 0;
+    }
+    len[e] = sum;
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int at = 0;
+    for (int e = 0; e < E; ++e) {
+      base[e] = at;
+      at += (len[e] + MOE_TILE_M - 1) / MOE_TILE_M * MOE_TILE_M;
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < E; e += nt) {
+    const int first = base[e];
+    for (int w = 0; w < n_waves; ++w) start[w * E + e] += first;
+    const int n = (len[e] + MOE_TILE_M - 1) / MOE_TILE_M;
+    for (int i = 0; i < n; ++i) tile_expert[first / MOE_TILE_M + i] = e;
+  }
+  __syncthreads();
+  moe_plan_pass(idx, p_lo, p_hi, cnt + wave * E, start + wave * E, true, slot_of_pair,
+                pair_of_slot);
 }
 
 extern "C" int kappai_moe_plan(const int* idx, int P, int E, int n_tiles, int* slot_of_pair,
@@ -144,14 +193,19 @@ extern "C" int kappai_moe_plan(const int* idx, int P, int E, int n_tiles, int* s
   if (P <= 0) return 0;
   if (E < 1 || E > 4096 || n_tiles < P / MOE_TILE_M + (E < P ? E : P))
     return (int)hipErrorInvalidValue;
-  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(WAVE), 2 * (size_t)E * sizeof(int), stream,
-                     idx, P, E, n_tiles, slot_of_pair, pair_of_slot, tile_expert);
+  // as many waves as have 64 pairs each and as the counters of fit into 48 KB of LDS
+  int n_waves = (P + WAVE - 1) / WAVE;
+  if (n_waves > MOE_PLAN_MAX_WAVES) n_waves = MOE_PLAN_MAX_WAVES;
+  while (n_waves > 1 && (size_t)(2 * n_waves + 2) * E * sizeof(int) > 48 * 1024) --n_waves;
+  const size_t lds = (size_t)(2 * n_waves + 2) * E * sizeof(int);
+  hipLaunchKernelGGL(moe_plan_kernel, dim3(1), dim3(n_waves * WAVE), lds, stream, idx, P, E,
+                     n_tiles, n_waves, slot_of_pair, pair_of_slot, tile_expert);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
 __device__ __forceinline__ float silu_exact(float g) { return g / (1.0f + expf(-g)); }
 
-// A tile of MOE_TILE_M slots of one expert times MOE_TILE_N rows of its matrix, float sums on
+// Half a tile (MOE_HALF_M slots) of one expert times MOE_TILE_N rows of its matrix, float sums on
 // the vector units (this is the 32-bit path, and the path of any shape).  GATED: the rows are
 // gathered from x by pair / top, two matrices, out = silu(g) * u in T; else the rows are the
 // slots of `a` themselves and out is float.
@@ -160,16 +214,16 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_gemm_kernel(
     const T* __restrict__ a, int lda, const T* __restrict__ w0, const T* __restrict__ w1, int N,
     int K, const int* __restrict__ tile_expert, const int* __restrict__ pair_of_slot, int top,
     void* __restrict__ out_v) {
-  const int tile = blockIdx.x;
+  const int tile = blockIdx.x / 2, slot0 = blockIdx.x * MOE_HALF_M;
   const int e = tile_expert[tile];
   if (e < 0) return;
-  __shared__ float As[MOE_TILE_K][MOE_TILE_M + 1];
+  __shared__ float As[MOE_TILE_K][MOE_HALF_M + 1];
   __shared__ float W0s[MOE_TILE_K][MOE_TILE_N + 1];
   __shared__ float W1s[GATED ? MOE_TILE_K : 1][MOE_TILE_N + 1];
-  __shared__ int src_row[MOE_TILE_M];
+  __shared__ int src_row[MOE_HALF_M];
   const int tid = threadIdx.x;
-  if (tid < MOE_TILE_M) {
-    const int slot = tile * MOE_TILE_M + tid;
+  if (tid < MOE_HALF_M) {
+    const int slot = slot0 + tid;
     const int pair = pair_of_slot[slot];
     src_row[tid] = pair < 0 ? -1 : (GATED ? pair / top : slot);
   }
@@ -217,7 +271,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_gemm_kernel(
   for (int i = 0; i < 2; ++i) {
     const int m = 2 * ty + i;
     if (src_row[m] < 0) continue;
-    const size_t slot = (size_t)tile * MOE_TILE_M + m;
+    const size_t slot = (size_t)slot0 + m;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx + 16 * j;
@@ -235,7 +289,7 @@ extern "C" int kappai_moe_gemm(const void* a, int lda, const void* w0, const voi
                                int n_tiles, void* out, int gated, int is_bf16,
                                hipStream_t stream) {
   if (n_tiles <= 0) return 0;
-  const dim3 grid(n_tiles, (N + MOE_TILE_N - 1) / MOE_TILE_N);
+  const dim3 grid(n_tiles * (MOE_TILE_M / MOE_HALF_M), (N + MOE_TILE_N - 1) / MOE_TILE_N);
   if (grid.y > 65535) return (int)hipErrorInvalidValue;
 #define MOE_GEMM_LAUNCH(TT, G)                                                                  \
   hipLaunchKernelGGL((moe_gemm_kernel<TT, G>), grid, dim3(MOE_THREADS), 0, stream, (const TT*)a, \
@@ -246,6 +300,137 @@ extern "C" int kappai_moe_gemm(const void* a, int lda, const void* w0, const voi
     if (gated) MOE_GEMM_LAUNCH(float, 1); else MOE_GEMM_LAUNCH(float, 0);
   }
 #undef MOE_GEMM_LAUNCH
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
+// The same products in bfloat16 on the matrix cores (v_mfma_f32_16x16x32_bf16).  A block owns a
+// tile of 64 slots (four row tiles of 16) and 4 waves x NT column tiles of 16 rows of the
+// expert's matrices; a wave streams its rows of W (and of the second matrix when GATED) and the
+// tile's activation rows straight from memory into registers, 16 bytes a lane, the next step of
+// 32 of K on its way while this one is multiplied.  Lane l holds row l % 16 of a fragment and the eight values of K from
+// 8 (l / 16); of a result tile it holds column l % 16 and the rows 4 (l / 16) .. + 3.
+// K must be a multiple of 8 and every row 16-byte aligned.
+// ---------------------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 moe_bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float moe_f32x4_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t moe_u32x4_t;
+
+#define MOE_MFMA_WAVES 4
+
+template <int GATED, int NT>
+__global__ __launch_bounds__(MOE_MFMA_WAVES * WAVE) void moe_gemm_mfma_kernel(
+    const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w0,
+    const bf16_t* __restrict__ w1, int N, int K, const int* __restrict__ tile_expert,
+    const int* __restrict__ pair_of_slot, int top, void* __restrict__ out_v) {
+  constexpr int MT = MOE_TILE_M / 16;
+  constexpr int NG = GATED ? 2 : 1;
+  const int tile = blockIdx.x;
+  const int e = tile_expert[tile];
+  if (e < 0) return;
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  const int col = lane % 16, kg = 8 * (lane / 16);
+  const int n0 = (blockIdx.y * MOE_MFMA_WAVES + wave) * 16 * NT;
+  if (n0 >= N) return;
+  const bf16_t* arow[MT];
+  bool a_ok[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int slot = tile * MOE_TILE_M + t * 16 + col;
+    const int pair = pair_of_slot[slot];
+    a_ok[t] = pair >= 0;
+    const int r = pair < 0 ? 0 : (GATED ? pair / top : slot);
+    arow[t] = a + (size_t)r * lda + kg;
+  }
+  const bf16_t* wrow[NG][NT];
+  bool w_ok[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int n = n0 + 16 * j + col;
+    w_ok[j] = n < N;
+    const size_t at = ((size_t)e * N + (w_ok[j] ? n : 0)) * K + kg;
+    wrow[0][j] = w0 + at;
+    if (GATED) wrow[1][j] = w1 + at;
+  }
+  moe_f32x4_t acc[NG][NT][MT];
+#pragma unroll
+  for (int g = 0; g < NG; ++g)
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int t = 0; t < MT; ++t) acc[g][j][t] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
+  const moe_u32x4_t zero = {0u, 0u, 0u, 0u};
+  // the loads of the next 32 of K are on their way while this step's are multiplied
+  moe_u32x4_t av[2][MT], wv[2][NG][NT];
+  auto load = [&](int buf, int gk) {
+    const bool kin = gk + kg < K;
+#pragma unroll
+    for (int t = 0; t < MT; ++t)
+      av[buf][t] = (kin && a_ok[t]) ? *reinterpret_cast<const moe_u32x4_t*>(arow[t] + gk) : zero;
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+        wv[buf][g][j] = (kin && w_ok[j])
+                            ? *reinterpret_cast<const moe_u32x4_t*>(wrow[g][j] + gk) : zero;
+  };
+  auto multiply = [&](int buf) {
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+          acc[g][j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+              __builtin_bit_cast(moe_bf16x8_t, av[buf][t]),
+              __builtin_bit_cast(moe_bf16x8_t, wv[buf][g][j]), acc[g][j][t], 0, 0, 0);
+  };
+  load(0, 0);
+  for (int k = 0; k < K; k += 64) {
+    load(1, k + 32);
+    multiply(0);
+    load(0, k + 64);
+    multiply(1);
+  }
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int m = t * 16 + 4 * (lane / 16) + v;
+      const size_t slot = (size_t)tile * MOE_TILE_M + m;
+      if (pair_of_slot[slot] < 0) continue;
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const int n = n0 + 16 * j + col;
+        if (n >= N) continue;
+        if (GATED)
+          ((bf16_t*)out_v)[slot * N + n] =
+              f32_to_bf16(silu_exact(acc[0][j][t][v]) * acc[GATED ? 1 : 0][j][t][v]);
+        else
+          ((float*)out_v)[slot * N + n] = acc[0][j][t][v];
+      }
+    }
+}
+
+extern "C" int kappai_moe_gemm_mfma(const void* a, int lda, const void* w0, const void* w1, int N,
+                                    int K, const int* tile_expert, const int* pair_of_slot,
+                                    int top, int n_tiles, void* out, int gated,
+                                    hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if ((K % 8) || (lda % 8) || ((uintptr_t)a % 16) || ((uintptr_t)w0 % 16) || ((uintptr_t)w1 % 16))
+    return (int)hipErrorInvalidValue;
+  const dim3 block(MOE_MFMA_WAVES * WAVE);
+  if (gated) {
+    const dim3 grid(n_tiles, (N + 16 * 2 * MOE_MFMA_WAVES - 1) / (16 * 2 * MOE_MFMA_WAVES));
+    hipLaunchKernelGGL((moe_gemm_mfma_kernel<1, 2>), grid, block, 0, stream, (const bf16_t*)a, lda,
+                       (const bf16_t*)w0, (const bf16_t*)w1, N, K, tile_expert, pair_of_slot, top,
+                       out);
+  } else {
+    const dim3 grid(n_tiles, (N + 16 * 4 * MOE_MFMA_WAVES - 1) / (16 * 4 * MOE_MFMA_WAVES));
+    hipLaunchKernelGGL((moe_gemm_mfma_kernel<0, 4>), grid, block, 0, stream, (const bf16_t*)a, lda,
+                       (const bf16_t*)w0, (const bf16_t*)w1, N, K, tile_expert, pair_of_slot, top,
+                       out);
+  }
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 

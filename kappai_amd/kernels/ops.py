@@ -1224,6 +1224,47 @@ def canon_conv(h: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, row_pos
     return out
 
 
+def add_group_rmsnorm_canon_step(resid: torch.Tensor, delta: Optional[torch.Tensor],
+                                 weight: torch.Tensor, eps: float, groups: int,
+                                 taps: torch.Tensor, state: torch.Tensor, row_pos: torch.Tensor,
+                                 seg_slot: torch.Tensor, out_dtype) -> torch.Tensor:
+    """``add_group_rmsnorm`` and ``canon_conv`` in one kernel for a step whose every segment is a
+    single row (row t is segment t): the residual gets the sum, the state its shift."""
+    _gpu("resid", resid, F32)
+    _gpu("weight", weight, F32)
+    _gpu("taps", taps, F32)
+    _gpu("state", state, F32)
+    _gpu("row_pos", row_pos, I32)
+    _gpu("seg_slot", seg_slot, I32)
+    T, D = resid.shape
+    n = taps.shape[1]
+    _need(weight.shape == (D,) and groups >= 1 and D % groups == 0 and (D + groups) * 4 <= 65536,
+          lambda: f"add_group_rmsnorm_canon_step: a width of {D} in {groups} groups")
+    _need(taps.shape[0] == D and 1 <= n <= CANON_MAX_TAPS and state.dim() == 3
+          and tuple(state.shape[1:]) == (n - 1, D),
+          lambda: f"add_group_rmsnorm_canon_step: taps {tuple(taps.shape)}, state "
+                  f"{tuple(state.shape)}")
+    _need(row_pos.shape[0] == T and seg_slot.shape[0] == T,
+          "add_group_rmsnorm_canon_step: one row a segment is needed")
+    kind, n_part = 0, 0
+    if delta is not None:
+        _gpu("delta", delta, (F32, BF16))
+        if delta.dim() == 3:
+            _need(delta.dtype == F32 and tuple(delta.shape[1:]) == (T, D),
+                  lambda: f"add_group_rmsnorm_canon_step: partial sums {tuple(delta.shape)}")
+            kind, n_part = 2, delta.shape[0]
+        else:
+            _need(tuple(delta.shape) == (T, D), "add_group_rmsnorm_canon_step: delta's shape")
+            kind, n_part = (1, 0) if delta.dtype == BF16 else (2, 1)
+    out = torch.empty((T, D), dtype=out_dtype, device=resid.device)
+    check(library("groupnorm").kappai_add_group_rmsnorm_canon_step(
+        _ptr(resid), _ptr(delta), _c_int(kind), _c_int(n_part), _c_int(T), _c_int(D),
+        _ptr(weight), _c_float(eps), _c_int(groups), _ptr(taps), _ptr(state), _ptr(row_pos),
+        _ptr(seg_slot), _c_int(n), _ptr(out), _c_int(_is_bf16(out_dtype)), _stream()),
+        "add_group_rmsnorm_canon_step")
+    return out
+
+
 def scale_add_positions(x: torch.Tensor, scale: float, table: torch.Tensor,
                         row_pos: torch.Tensor) -> None:
     """``x[t] = x[t] * scale + table[row_pos[t]]`` in place on float32 rows.  The caller keeps
@@ -1259,24 +1300,22 @@ def glu(gate_up: torch.Tensor, kind: int) -> torch.Tensor:
 # ---------------------------------------------------------------------------------------
 # minGRU
 # ---------------------------------------------------------------------------------------
-def mingru_chunk_rows() -> int:
-    return int(library("mingru").kappai_mingru_chunk_rows())
-
-
 def mingru_scan(proj: torch.Tensor, state: torch.Tensor, seg_start: torch.Tensor,
                 seg_pos0: torch.Tensor, seg_slot: torch.Tensor, out_dtype,
                 chunks: Optional[torch.Tensor] = None,
                 seg_chunk0: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """The minGRU recurrence over float32 projections [T, 3W] = (update gate | candidate | output
-    gate, biases added): ``S = (1 - z) S + z c`` with ``z = sigmoid``, ``c = u + 1/2`` for
+    """The minGRU recurrence over projections [T, 3W] = (update gate | candidate | output gate,
+    biases added; float32, or bfloat16 when the output is bfloat16 too): ``S = (1 - z) S + z c`` with ``z = sigmoid``, ``c = u + 1/2`` for
     ``u >= 0`` and ``sigmoid(u)`` below, output ``S * silu(g)`` [T, W] in ``out_dtype``.  ``state``
     [slots, W] float32 is read (unless the segment starts at position 0) and left at the
     segment's last row.  ``chunks`` [n, 3] = (segment, first row, rows) with ``seg_chunk0`` [S + 1]:
     long segments are scanned chunk by chunk in three passes."""
-    _gpu("proj", proj, F32)
+    _gpu("proj", proj, (F32, BF16))
     _gpu("state", state, F32)
     T = proj.shape[0]
     _need(proj.dim() == 2 and proj.shape[1] % 3 == 0, lambda: f"mingru_scan: {tuple(proj.shape)}")
+    _need(proj.dtype == F32 or out_dtype == BF16,
+          "mingru_scan: bfloat16 projections give bfloat16 outputs")
     W = proj.shape[1] // 3
     _need(state.dim() == 2 and state.shape[1] == W,
           lambda: f"mingru_scan: state {tuple(state.shape)} for a width of {W}")
@@ -1293,9 +1332,10 @@ def mingru_scan(proj: torch.Tensor, state: torch.Tensor, seg_start: torch.Tensor
         _need(chunks.dim() == 2 and chunks.shape[1] == 3 and seg_chunk0.shape[0] == S + 1,
               "mingru_scan: chunk tables do not fit")
         n_chunks = chunks.shape[0]
-        carry = torch.empty((n_chunks, 2, W), dtype=F32, device=proj.device)
+        carry = torch.empty((n_chunks, 3, W), dtype=F32, device=proj.device)
     check(library("mingru").kappai_mingru_scan(
-        _ptr(proj), _ptr(state), _ptr(seg_start), _ptr(seg_pos0), _ptr(seg_slot), _c_int(T),
+        _ptr(proj), _c_int(_is_bf16(proj.dtype)), _ptr(state), _ptr(seg_start), _ptr(seg_pos0),
+        _ptr(seg_slot), _c_int(T),
         _c_int(S), _c_int(W), _ptr(chunks), _ptr(seg_chunk0), _c_int(n_chunks), _ptr(carry),
         _ptr(out), _c_int(_is_bf16(out_dtype)), _stream()), "mingru_scan")
     return out
@@ -1408,6 +1448,14 @@ def moe_plan(experts: torch.Tensor, n_experts: int) -> MoePlan:
     return plan
 
 
+MOE_MFMA = True       # bfloat16 expert products on the matrix cores (False: the plain kernel)
+
+
+def _moe_on_matrix_cores(a: torch.Tensor, lda: int, K: int, *matrices) -> bool:
+    return (MOE_MFMA and a.dtype == BF16 and K % 8 == 0 and lda % 8 == 0
+            and a.data_ptr() % 16 == 0 and all(m.data_ptr() % 16 == 0 for m in matrices))
+
+
 def moe_experts_gated(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor,
                       plan: MoePlan) -> torch.Tensor:
     """``silu(x Wg[e]^T) * (x Wu[e]^T)`` for every slot of the plan ([slots, F], the dtype of
@@ -1419,6 +1467,12 @@ def moe_experts_gated(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor,
     _need(w_up.shape == w_gate.shape and x.shape[1] == D and x.stride(1) == 1,
           lambda: f"moe_experts_gated: x {tuple(x.shape)}, matrices {tuple(w_gate.shape)}")
     out = torch.empty((plan.n_tiles * plan.tile_rows, F), dtype=x.dtype, device=x.device)
+    if _moe_on_matrix_cores(x, x.stride(0), D, w_gate, w_up):
+        check(library("moe").kappai_moe_gemm_mfma(
+            _ptr(x), _c_int(x.stride(0)), _ptr(w_gate), _ptr(w_up), _c_int(F), _c_int(D),
+            _ptr(plan.tile_expert), _ptr(plan.pair_of_slot), _c_int(plan.top),
+            _c_int(plan.n_tiles), _ptr(out), _c_int(1), _stream()), "moe_gemm_mfma (gate, up)")
+        return out
     check(library("moe").kappai_moe_gemm(
         _ptr(x), _c_int(x.stride(0)), _ptr(w_gate), _ptr(w_up), _c_int(F), _c_int(D),
         _ptr(plan.tile_expert), _ptr(plan.pair_of_slot), _c_int(plan.top), _c_int(plan.n_tiles),
@@ -1434,6 +1488,12 @@ def moe_experts_down(act: torch.Tensor, w_down: torch.Tensor, plan: MoePlan) -> 
     _need(tuple(act.shape) == (plan.n_tiles * plan.tile_rows, F),
           lambda: f"moe_experts_down: act {tuple(act.shape)}, matrices {tuple(w_down.shape)}")
     out = torch.empty((act.shape[0], D), dtype=F32, device=act.device)
+    if _moe_on_matrix_cores(act, F, F, w_down):
+        check(library("moe").kappai_moe_gemm_mfma(
+            _ptr(act), _c_int(F), _ptr(w_down), _vp(0), _c_int(D), _c_int(F),
+            _ptr(plan.tile_expert), _ptr(plan.pair_of_slot), _c_int(plan.top),
+            _c_int(plan.n_tiles), _ptr(out), _c_int(0), _stream()), "moe_gemm_mfma (down)")
+        return out
     check(library("moe").kappai_moe_gemm(
         _ptr(act), _c_int(F), _ptr(w_down), _vp(0), _c_int(D), _c_int(F),
         _ptr(plan.tile_expert), _ptr(plan.pair_of_slot), _c_int(plan.top), _c_int(plan.n_tiles),

@@ -175,6 +175,8 @@ class ConvInputBlock(Block):
         delta = summed_delta(norm, delta)
         if conv is None:
             return norm.add_norm(resid, delta)
+        if batch.max_segment_rows == 1 and hasattr(norm, "add_norm_conv_step"):
+            return norm.add_norm_conv_step(resid, delta, conv, batch, state)    # decode: one kernel
         if getattr(norm, "takes_out_dtype", False):
             h = norm.add_norm(resid, delta, out_dtype=torch.float32)
         else:

@@ -39,6 +39,16 @@ class GroupRMSNorm(Norm):
                                          out_dtype or self.dtype, rows=rows,
                                          write_resid=rows is None)
 
+    def add_norm_conv_step(self, resid, delta, conv, batch, cache):
+        """The norm and the short convolution behind it (``parts.input_conv.ShortInputConv``) in
+        one kernel, for a step whose segments are single rows."""
+        if isinstance(delta, ops.Added):
+            delta = None
+        with profile.scope("rmsnorm"):
+            return ops.add_group_rmsnorm_canon_step(
+                resid, delta, self.weight, self.eps, self.groups, conv.taps, cache.state,
+                batch.row_pos, batch.seg_slot, conv.dtype)
+
     def weight_bytes(self) -> int:
         return self.width * 4
 

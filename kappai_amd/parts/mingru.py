@@ -3,7 +3,8 @@
 ``z = sigmoid(W_z h + b_z)``, ``u = W_x h + b_x``; the candidate is ``u + 1/2`` where ``u >= 0``
 and ``sigmoid(u)`` below; element by element ``S_t = (1 - z) S_(t-1) + z * candidate`` from a zero
 state; the output is ``W_o (S_t * silu(W_g h))``.  The three input products run as one; gates,
-candidates and the state are float32, the state a slot of ``inner`` floats a request.
+candidates and the state are float32 (computed from the products' results as they are stored), the state a slot
+of ``inner`` floats a request.
 """
 from __future__ import annotations
 
@@ -77,7 +78,9 @@ class MinGRU(Mixer):
     def forward(self, x, batch, cache, shared_cache: bool = False):
         if shared_cache:
             raise ValueError("a recurrent state cannot be read by another layer")
-        proj = self.gates.forward(x, out_dtype=torch.float32)
+        # (the products' results are stored in the compute dtype, as every other product's; what
+        # the recurrence makes of them is float32)
+        proj = self.gates.forward(x)
         chunked = batch.max_segment_rows > tuning.SCAN_CHUNKS_FROM_ROWS
         with profile.scope("scan"):
             y = ops.mingru_scan(proj, cache.state, batch.seg_start, batch.seg_pos0,

@@ -292,6 +292,14 @@ def canon_conv(h, taps, state, row_pos, row_seg, seg_start, seg_slot, out_dtype)
     return out.to(out_dtype)
 
 
+def add_group_rmsnorm_canon_step(resid, delta, weight, eps, groups, taps, state, row_pos, seg_slot,
+                                 out_dtype):
+    T = resid.shape[0]
+    h = add_group_rmsnorm(resid, delta, weight, eps, groups, F32)
+    ar = torch.arange(T + 1, dtype=torch.int32)
+    return canon_conv(h, taps, state, row_pos, ar[:T], ar, seg_slot, out_dtype)
+
+
 def scale_add_positions(x, scale, table, row_pos):
     x.mul_(scale).add_(table[row_pos.long()].to(F32))
 
@@ -309,6 +317,7 @@ def glu(gate_up, kind):
 # ---- minGRU ----------------------------------------------------------------------------------
 def mingru_scan(proj, state, seg_start, seg_pos0, seg_slot, out_dtype, chunks=None,
                 seg_chunk0=None):
+    proj = proj.to(F32)
     T, W = proj.shape[0], proj.shape[1] // 3
     out = torch.empty((T, W), dtype=F32)
     for s in range(seg_slot.shape[0]):
@@ -397,7 +406,7 @@ def moe_combine(y, weights, plan):
     return (y * weights[:, :, None]).sum(dim=1)
 
 
-ALL = ["add_group_rmsnorm", "canon_conv", "scale_add_positions", "glu", "mingru_scan", "diff_store",
+ALL = ["add_group_rmsnorm", "add_group_rmsnorm_canon_step", "canon_conv", "scale_add_positions", "glu", "mingru_scan", "diff_store",
        "diff_combine", "moe_route", "moe_plan", "moe_experts_gated", "moe_experts_down", "moe_combine",
        "embed_rows", "add_rmsnorm", "add_residual", "sum_partial_sums", "swiglu", "cast", "linear", "linear_swiglu",
        "interleave_gate_up", "shortconv", "linear_shortconv_step",

@@ -400,3 +400,29 @@ def test_greedy_generation_through_the_engine(model_dirs):
         assert eng.cache.num_free_slots == 3
         assert all(g.allocator.num_used == 0 for g in eng.cache.paged_groups)
         eng.shutdown()
+
+
+@pytest.mark.parametrize("taps,groups", [(4, 3), (1, 1), (2, 8)])
+def test_fused_decode_norm_and_convolution_equal_the_two_kernels(taps, groups):
+    """The one kernel of a decode step (residual sum, grouped norm, convolution, state shift)
+    against the norm kernel followed by the convolution's two, over several steps of three rows in
+    different slots, from position 0 on (NaN in the states before)."""
+    from kappai_amd.kernels import ops
+    D, B = 96, 3
+    w = (1 + 0.1 * torch.randn(D, generator=gen(30))).to(DEV)
+    tw = (torch.randn(D, taps, generator=gen(31)) * 0.4).to(DEV)
+    states = [torch.full((5, taps - 1, D), float("nan"), device=DEV) for _ in range(2)]
+    resid = [(torch.randn(B, D, generator=gen(32)) * 2).to(DEV) for _ in range(2)]
+    slots = torch.tensor([4, 0, 2], dtype=torch.int32, device=DEV)
+    ar = torch.arange(B + 1, dtype=torch.int32, device=DEV)
+    for step in range(7):
+        delta = torch.randn(B, D, generator=gen(40 + step)).to(BF16).to(DEV) if step else None
+        pos = torch.tensor([step, step, step], dtype=torch.int32, device=DEV)
+        fused = ops.add_group_rmsnorm_canon_step(resid[0], delta, w, 1e-5, groups, tw, states[0],
+                                                 pos, slots, F32)
+        h = ops.add_group_rmsnorm(resid[1], delta, w, 1e-5, groups, F32)
+        two = ops.canon_conv(h, tw, states[1], pos, ar[:B], ar, slots, F32)
+        assert torch.equal(fused, two) and torch.equal(resid[0], resid[1])
+        if step >= taps - 1:         # (before that the state's oldest places hold nothing yet)
+            used = slots.long()
+            assert torch.equal(states[0][used], states[1][used])
