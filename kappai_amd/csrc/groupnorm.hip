@@ -141,9 +141,12 @@ extern "C" int kappai_canon_conv(const float* h, const float* taps, float* state
 }
 
 // A step of single rows (every segment one decoded token): residual sum, norm, convolution and
-// the state's shift in one kernel, a block a row.  Row t is segment t; its history is all state.
+// the state's shift in one kernel, a block of 1024 threads a row (a thread has one or two columns
+// of the usual widths: what it loads, it loads at once).  Row t is segment t; its history is all
+// state.
+#define GN_STEP_THREADS 1024
 template <typename TO>
-__global__ __launch_bounds__(GN_THREADS) void add_group_rmsnorm_canon_step_kernel(
+__global__ __launch_bounds__(GN_STEP_THREADS) void add_group_rmsnorm_canon_step_kernel(
     float* __restrict__ resid, const void* __restrict__ delta, int delta_kind, int n_part,
     size_t part_stride, const float* __restrict__ w, float eps, int groups, int D,
     const float* __restrict__ taps, float* __restrict__ state, const int* __restrict__ row_pos,
@@ -152,7 +155,7 @@ __global__ __launch_bounds__(GN_THREADS) void add_group_rmsnorm_canon_step_kerne
   float* scale = row + D;
   const int r = blockIdx.x;
   float* x = resid + (size_t)r * D;
-  for (int i = threadIdx.x; i < D; i += GN_THREADS) {
+  for (int i = threadIdx.x; i < D; i += GN_STEP_THREADS) {
     float v = x[i];
     if (delta_kind == 1) {
       v += bf16_to_f32(((const bf16_t*)delta)[(size_t)r * D + i]);
@@ -166,7 +169,7 @@ __global__ __launch_bounds__(GN_THREADS) void add_group_rmsnorm_canon_step_kerne
   __syncthreads();
   const int gs = D / groups;
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  for (int g = wave; g < groups; g += GN_THREADS / WAVE) {
+  for (int g = wave; g < groups; g += GN_STEP_THREADS / WAVE) {
     float ss = 0.f;
     for (int i = lane; i < gs; i += WAVE) {
       const float v = row[g * gs + i];
@@ -178,7 +181,7 @@ __global__ __launch_bounds__(GN_THREADS) void add_group_rmsnorm_canon_step_kerne
   __syncthreads();
   const int pos = row_pos[r];
   float* st = state + (size_t)seg_slot[r] * (n_taps - 1) * D;
-  for (int c = threadIdx.x; c < D; c += GN_THREADS) {
+  for (int c = threadIdx.x; c < D; c += GN_STEP_THREADS) {
     // state[k] is the input n - 1 - k places back; everything is asked for before it is used
     float keep[CANON_MAX_TAPS], tw[CANON_MAX_TAPS];
 #pragma unroll
@@ -216,11 +219,11 @@ extern "C" int kappai_add_group_rmsnorm_canon_step(float* resid, const void* del
   if (lds > 64 * 1024) return (int)hipErrorInvalidValue;
   const size_t ps = (size_t)T * D;
   if (out_is_bf16)
-    hipLaunchKernelGGL(add_group_rmsnorm_canon_step_kernel<bf16_t>, dim3(T), dim3(GN_THREADS), lds,
+    hipLaunchKernelGGL(add_group_rmsnorm_canon_step_kernel<bf16_t>, dim3(T), dim3(GN_STEP_THREADS), lds,
                        stream, resid, delta, delta_kind, n_part, ps, w, eps, groups, D, taps, state,
                        row_pos, seg_slot, n_taps, (bf16_t*)out);
   else
-    hipLaunchKernelGGL(add_group_rmsnorm_canon_step_kernel<float>, dim3(T), dim3(GN_THREADS), lds,
+    hipLaunchKernelGGL(add_group_rmsnorm_canon_step_kernel<float>, dim3(T), dim3(GN_STEP_THREADS), lds,
                        stream, resid, delta, delta_kind, n_part, ps, w, eps, groups, D, taps, state,
                        row_pos, seg_slot, n_taps, (float*)out);
   KAPPAI_RETURN_LAUNCH_STATUS();

@@ -18,40 +18,61 @@
 
 extern "C" int kappai_moe_tile_rows() { return MOE_TILE_M; }
 
-#define MOE_ROUTE_GROUP 8       // experts whose sums a lane carries side by side
+#define MOE_ROUTE_GROUP 16      // experts whose sums a thread carries side by side
 
-template <typename T>
+// A block a row.  The threads stride over the row four columns at a time (one column at a time
+// when the width or an address does not allow 16-byte loads), each with the sums of a group of
+// experts, whose loads are all asked for before the first is used; the waves' sums meet in LDS
+// and are added in the order of the waves.  Then the first wave chooses.
+template <typename T, int VEC>
 __global__ __launch_bounds__(MOE_THREADS) void moe_route_kernel(
     const T* __restrict__ x, int ldx, const float* __restrict__ router, int n_rows, int D, int E,
     int top, int* __restrict__ idx, float* __restrict__ wts) {
-  extern __shared__ float logits_all[];
+  extern __shared__ float route_lds[];
+  constexpr int NW = MOE_THREADS / WAVE;
+  float* logits = route_lds;                       // [E]
+  float* part = route_lds + E;                     // [MOE_ROUTE_GROUP][NW]
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
-  const int row_raw = blockIdx.x * (MOE_THREADS / WAVE) + wave;
-  const int row = row_raw < n_rows ? row_raw : n_rows - 1;
-  float* logits = logits_all + wave * E;
+  const int row = blockIdx.x;
   const T* xr = x + (size_t)row * ldx;
-  // a wave a row; the lanes stride over the row, each with the sums of a group of experts, so
-  // that the loads of a pass do not wait for one another
   for (int e0 = 0; e0 < E; e0 += MOE_ROUTE_GROUP) {
     float acc[MOE_ROUTE_GROUP];
 #pragma unroll
     for (int j = 0; j < MOE_ROUTE_GROUP; ++j) acc[j] = 0.f;
-#pragma unroll 4
-    for (int c = lane; c < D; c += WAVE) {
-      const float xv = to_f32(xr[c]);
+    for (int c = threadIdx.x * VEC; c < D; c += MOE_THREADS * VEC) {
+      float xv[VEC], rv[MOE_ROUTE_GROUP][VEC];
 #pragma unroll
       for (int j = 0; j < MOE_ROUTE_GROUP; ++j) {
-        const int e = min(e0 + j, E - 1);
-        acc[j] = fmaf(xv, router[(size_t)e * D + c], acc[j]);
+        const float* r = router + (size_t)min(e0 + j, E - 1) * D + c;
+        if (VEC == 4) {
+          const float4 v = *reinterpret_cast<const float4*>(r);
+          rv[j][0] = v.x; rv[j][VEC > 1 ? 1 : 0] = v.y; rv[j][VEC > 2 ? 2 : 0] = v.z;
+          rv[j][VEC > 3 ? 3 : 0] = v.w;
+        } else {
+          rv[j][0] = r[0];
+        }
       }
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) xv[i] = to_f32(xr[c + i]);
+#pragma unroll
+      for (int j = 0; j < MOE_ROUTE_GROUP; ++j)
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) acc[j] = fmaf(xv[i], rv[j][i], acc[j]);
     }
 #pragma unroll
     for (int j = 0; j < MOE_ROUTE_GROUP; ++j) {
       const float sum = wave_sum(acc[j]);
-      if (lane == 0 && e0 + j < E) logits[e0 + j] = sum;
+      if (lane == 0) part[j * NW + wave] = sum;
     }
+    __syncthreads();
+    if (threadIdx.x < MOE_ROUTE_GROUP && e0 + threadIdx.x < E) {
+      float sum = part[threadIdx.x * NW];
+      for (int w = 1; w < NW; ++w) sum += part[threadIdx.x * NW + w];
+      logits[e0 + threadIdx.x] = sum;
+    }
+    __syncthreads();
   }
-  __syncthreads();
+  if (wave != 0) return;
   float cv[MOE_MAX_TOP];
   int ci[MOE_MAX_TOP];
 #pragma unroll
@@ -67,12 +88,13 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_route_kernel(
       const int who = -wave_max(best == m ? -at : -0x7fffffff);
       cv[k] = m;
       ci[k] = who;
-      __syncthreads();
+      __builtin_amdgcn_wave_barrier();
       if (lane == 0 && who < E) logits[who] = -INFINITY;
-      __syncthreads();
+      __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+      __builtin_amdgcn_wave_barrier();
     }
   }
-  if (lane == 0 && row_raw < n_rows) {
+  if (lane == 0) {
     float sum = 0.f;
 #pragma unroll
     for (int k = 0; k < MOE_MAX_TOP; ++k)
@@ -90,15 +112,17 @@ extern "C" int kappai_moe_route(const void* x, int ldx, int x_is_bf16, const flo
                                 int D, int E, int top, int* idx, float* wts, hipStream_t stream) {
   if (T <= 0) return 0;
   if (top < 1 || top > MOE_MAX_TOP || top > E || E > 4096) return (int)hipErrorInvalidValue;
-  const int waves = MOE_THREADS / WAVE;
-  const dim3 grid((T + waves - 1) / waves);
-  const size_t lds = (size_t)waves * E * sizeof(float);
-  if (x_is_bf16)
-    hipLaunchKernelGGL(moe_route_kernel<bf16_t>, grid, dim3(MOE_THREADS), lds, stream,
-                       (const bf16_t*)x, ldx, router, T, D, E, top, idx, wts);
-  else
-    hipLaunchKernelGGL(moe_route_kernel<float>, grid, dim3(MOE_THREADS), lds, stream,
-                       (const float*)x, ldx, router, T, D, E, top, idx, wts);
+  const size_t lds = (size_t)(E + MOE_ROUTE_GROUP * (MOE_THREADS / WAVE)) * sizeof(float);
+  const bool vec = D % 4 == 0 && (uintptr_t)router % 16 == 0;
+#define MOE_ROUTE_LAUNCH(TT, V)                                                                 \
+  hipLaunchKernelGGL((moe_route_kernel<TT, V>), dim3(T), dim3(MOE_THREADS), lds, stream,          \
+                     (const TT*)x, ldx, router, T, D, E, top, idx, wts)
+  if (x_is_bf16) {
+    if (vec) MOE_ROUTE_LAUNCH(bf16_t, 4); else MOE_ROUTE_LAUNCH(bf16_t, 1);
+  } else {
+    if (vec) MOE_ROUTE_LAUNCH(float, 4); else MOE_ROUTE_LAUNCH(float, 1);
+  }
+#undef MOE_ROUTE_LAUNCH
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
@@ -310,7 +334,8 @@ extern "C" int kappai_moe_gemm(const void* a, int lda, const void* w0, const voi
 // tile's activation rows straight from memory into registers, 16 bytes a lane, the next step of
 // 32 of K on its way while this one is multiplied.  Lane l holds row l % 16 of a fragment and the eight values of K from
 // 8 (l / 16); of a result tile it holds column l % 16 and the rows 4 (l / 16) .. + 3.
-// K must be a multiple of 8 and every row 16-byte aligned.
+// K must be a multiple of 8 and every row 16-byte aligned (fragment order: K a multiple of 32,
+// the matrices' rows a multiple of 16).
 // ---------------------------------------------------------------------------------------
 typedef __attribute__((ext_vector_type(8))) __bf16 moe_bf16x8_t;
 typedef __attribute__((ext_vector_type(4))) float moe_f32x4_t;
@@ -318,7 +343,10 @@ typedef __attribute__((ext_vector_type(4))) uint32_t moe_u32x4_t;
 
 #define MOE_MFMA_WAVES 4
 
-template <int GATED, int NT>
+// WF: the experts' matrices lie in fragment order (the host arranges them once): the 16 rows x
+// 32 of K that a matrix instruction takes are 1 KB in a row, lane after lane, tile (row tile,
+// step of K) after tile, so that a wave's load is one piece of memory instead of sixteen.
+template <int GATED, int NT, int U, bool WF>
 __global__ __launch_bounds__(MOE_MFMA_WAVES * WAVE) void moe_gemm_mfma_kernel(
     const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w0,
     const bf16_t* __restrict__ w1, int N, int K, const int* __restrict__ tile_expert,
@@ -348,7 +376,9 @@ __global__ __launch_bounds__(MOE_MFMA_WAVES * WAVE) void moe_gemm_mfma_kernel(
   for (int j = 0; j < NT; ++j) {
     const int n = n0 + 16 * j + col;
     w_ok[j] = n < N;
-    const size_t at = ((size_t)e * N + (w_ok[j] ? n : 0)) * K + kg;
+    const size_t at = WF ? (size_t)e * N * K + (size_t)((w_ok[j] ? n : 0) / 16) * (K / 32) * 512 +
+                               lane * 8
+                         : ((size_t)e * N + (w_ok[j] ? n : 0)) * K + kg;
     wrow[0][j] = w0 + at;
     if (GATED) wrow[1][j] = w1 + at;
   }
@@ -360,36 +390,45 @@ __global__ __launch_bounds__(MOE_MFMA_WAVES * WAVE) void moe_gemm_mfma_kernel(
 #pragma unroll
       for (int t = 0; t < MT; ++t) acc[g][j][t] = moe_f32x4_t{0.f, 0.f, 0.f, 0.f};
   const moe_u32x4_t zero = {0u, 0u, 0u, 0u};
-  // the loads of the next 32 of K are on their way while this step's are multiplied
-  moe_u32x4_t av[2][MT], wv[2][NG][NT];
-  auto load = [&](int buf, int gk) {
-    const bool kin = gk + kg < K;
+  // the loads of the next U steps of 32 of K are on their way while these are multiplied
+  moe_u32x4_t av[2][U][MT], wv[2][U][NG][NT];
+  auto load = [&](int buf, int k0) {
 #pragma unroll
-    for (int t = 0; t < MT; ++t)
-      av[buf][t] = (kin && a_ok[t]) ? *reinterpret_cast<const moe_u32x4_t*>(arow[t] + gk) : zero;
+    for (int u = 0; u < U; ++u) {
+      const int gk = k0 + 32 * u;
+      const bool kin = gk + kg < K;
 #pragma unroll
-    for (int g = 0; g < NG; ++g)
+      for (int t = 0; t < MT; ++t)
+        av[buf][u][t] =
+            (kin && a_ok[t]) ? *reinterpret_cast<const moe_u32x4_t*>(arow[t] + gk) : zero;
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
-        wv[buf][g][j] = (kin && w_ok[j])
-                            ? *reinterpret_cast<const moe_u32x4_t*>(wrow[g][j] + gk) : zero;
+      for (int g = 0; g < NG; ++g)
+#pragma unroll
+        for (int j = 0; j < NT; ++j)
+          wv[buf][u][g][j] = (kin && w_ok[j])
+                                 ? *reinterpret_cast<const moe_u32x4_t*>(
+                                       wrow[g][j] + (WF ? (size_t)(gk / 32) * 512 : (size_t)gk))
+                                 : zero;
+    }
   };
   auto multiply = [&](int buf) {
 #pragma unroll
-    for (int g = 0; g < NG; ++g)
+    for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int j = 0; j < NT; ++j)
+      for (int g = 0; g < NG; ++g)
 #pragma unroll
-        for (int t = 0; t < MT; ++t)
-          acc[g][j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-              __builtin_bit_cast(moe_bf16x8_t, av[buf][t]),
-              __builtin_bit_cast(moe_bf16x8_t, wv[buf][g][j]), acc[g][j][t], 0, 0, 0);
+        for (int j = 0; j < NT; ++j)
+#pragma unroll
+          for (int t = 0; t < MT; ++t)
+            acc[g][j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                __builtin_bit_cast(moe_bf16x8_t, av[buf][u][t]),
+                __builtin_bit_cast(moe_bf16x8_t, wv[buf][u][g][j]), acc[g][j][t], 0, 0, 0);
   };
   load(0, 0);
-  for (int k = 0; k < K; k += 64) {
-    load(1, k + 32);
+  for (int k = 0; k < K; k += 64 * U) {
+    load(1, k + 32 * U);
     multiply(0);
-    load(0, k + 64);
+    load(0, k + 64 * U);
     multiply(1);
   }
 #pragma unroll
@@ -412,25 +451,31 @@ __global__ __launch_bounds__(MOE_MFMA_WAVES * WAVE) void moe_gemm_mfma_kernel(
     }
 }
 
+// `few`: a step of few rows (decoding), where a tile holds a row or two and the kernel streams
+// the experts' matrices: one column tile a wave (twice the blocks) and two steps of K a load.
 extern "C" int kappai_moe_gemm_mfma(const void* a, int lda, const void* w0, const void* w1, int N,
                                     int K, const int* tile_expert, const int* pair_of_slot,
-                                    int top, int n_tiles, void* out, int gated,
-                                    hipStream_t stream) {
+                                    int top, int n_tiles, void* out, int gated, int few,
+                                    int w_frag, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if ((K % 8) || (lda % 8) || ((uintptr_t)a % 16) || ((uintptr_t)w0 % 16) || ((uintptr_t)w1 % 16))
     return (int)hipErrorInvalidValue;
+  if (w_frag && ((K % 32) || (N % 16))) return (int)hipErrorInvalidValue;
   const dim3 block(MOE_MFMA_WAVES * WAVE);
+#define MOE_MFMA_LAUNCH(G, NT_, U_)                                                              \
+  if (w_frag) MOE_MFMA_LAUNCH_WF(G, NT_, U_, true); else MOE_MFMA_LAUNCH_WF(G, NT_, U_, false)
+#define MOE_MFMA_LAUNCH_WF(G, NT_, U_, WF_)                                                      \
+  hipLaunchKernelGGL((moe_gemm_mfma_kernel<G, NT_, U_, WF_>),                                    \
+                     dim3(n_tiles, (N + 16 * NT_ * MOE_MFMA_WAVES - 1) / (16 * NT_ * MOE_MFMA_WAVES)), \
+                     block, 0, stream, (const bf16_t*)a, lda, (const bf16_t*)w0, (const bf16_t*)w1, \
+                     N, K, tile_expert, pair_of_slot, top, out)
   if (gated) {
-    const dim3 grid(n_tiles, (N + 16 * 2 * MOE_MFMA_WAVES - 1) / (16 * 2 * MOE_MFMA_WAVES));
-    hipLaunchKernelGGL((moe_gemm_mfma_kernel<1, 2>), grid, block, 0, stream, (const bf16_t*)a, lda,
-                       (const bf16_t*)w0, (const bf16_t*)w1, N, K, tile_expert, pair_of_slot, top,
-                       out);
+    if (few) { MOE_MFMA_LAUNCH(1, 1, 2); } else { MOE_MFMA_LAUNCH(1, 4, 1); }
   } else {
-    const dim3 grid(n_tiles, (N + 16 * 4 * MOE_MFMA_WAVES - 1) / (16 * 4 * MOE_MFMA_WAVES));
-    hipLaunchKernelGGL((moe_gemm_mfma_kernel<0, 4>), grid, block, 0, stream, (const bf16_t*)a, lda,
-                       (const bf16_t*)w0, (const bf16_t*)w1, N, K, tile_expert, pair_of_slot, top,
-                       out);
+    if (few) { MOE_MFMA_LAUNCH(0, 2, 2); } else { MOE_MFMA_LAUNCH(0, 4, 1); }
   }
+#undef MOE_MFMA_LAUNCH
+#undef MOE_MFMA_LAUNCH_WF
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 

@@ -1451,6 +1451,45 @@ def moe_plan(experts: torch.Tensor, n_experts: int) -> MoePlan:
 MOE_MFMA = True       # bfloat16 expert products on the matrix cores (False: the plain kernel)
 
 
+MOE_FEW_PAIRS = 256   # up to this many (row, choice) pairs the expert kernels stream the matrices
+
+
+class ExpertFragments:
+    """The matrices of a mixture's experts [E, N, K] in the order the matrix-core kernel loads
+    them: every 16 rows x 32 columns as one piece of 1 KB, lane after lane (lane = row + 16 *
+    (column // 8)), the pieces of a row tile one after the other.  N a multiple of 16, K of 32."""
+
+    def __init__(self, data: torch.Tensor, shape):
+        self.data, self.shape = data, tuple(shape)
+        self.dtype, self.device = data.dtype, data.device
+
+    @staticmethod
+    def fits(weight: torch.Tensor) -> bool:
+        return (weight.dtype == BF16 and weight.dim() == 3 and weight.shape[1] % 16 == 0
+                and weight.shape[2] % 32 == 0)
+
+    @classmethod
+    def of(cls, weight: torch.Tensor) -> "ExpertFragments":
+        E, N, K = weight.shape
+        w = weight.reshape(E, N // 16, 16, K // 32, 4, 8).permute(0, 1, 3, 4, 2, 5)
+        return cls(w.contiguous(), (E, N, K))
+
+    def data_ptr(self) -> int:
+        return self.data.data_ptr()
+
+    def element_size(self) -> int:
+        return self.data.element_size()
+
+
+def _moe_matrix(w):
+    """(tensor for the checks, 1 if it lies in fragment order)"""
+    return (w.data, 1) if isinstance(w, ExpertFragments) else (w, 0)
+
+
+def _moe_few(plan) -> int:
+    return 1 if plan.slot_of_pair.shape[0] <= MOE_FEW_PAIRS else 0
+
+
 def _moe_on_matrix_cores(a: torch.Tensor, lda: int, K: int, *matrices) -> bool:
     return (MOE_MFMA and a.dtype == BF16 and K % 8 == 0 and lda % 8 == 0
             and a.data_ptr() % 16 == 0 and all(m.data_ptr() % 16 == 0 for m in matrices))
@@ -1461,17 +1500,23 @@ def moe_experts_gated(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor,
     """``silu(x Wg[e]^T) * (x Wu[e]^T)`` for every slot of the plan ([slots, F], the dtype of
     ``x``; empty slots are left unwritten).  ``w_gate``, ``w_up``: [E, F, D]."""
     _gpu("x", x, (F32, BF16), contiguous=False)
+    E, F, D = w_gate.shape
+    (w_gate, frag), (w_up, frag_up) = _moe_matrix(w_gate), _moe_matrix(w_up)
     _gpu("w_gate", w_gate, x.dtype)
     _gpu("w_up", w_up, x.dtype)
-    E, F, D = w_gate.shape
-    _need(w_up.shape == w_gate.shape and x.shape[1] == D and x.stride(1) == 1,
-          lambda: f"moe_experts_gated: x {tuple(x.shape)}, matrices {tuple(w_gate.shape)}")
+    _need(w_up.shape == w_gate.shape and frag == frag_up and x.shape[1] == D
+          and x.stride(1) == 1,
+          lambda: f"moe_experts_gated: x {tuple(x.shape)}, matrices {(E, F, D)}")
     out = torch.empty((plan.n_tiles * plan.tile_rows, F), dtype=x.dtype, device=x.device)
-    if _moe_on_matrix_cores(x, x.stride(0), D, w_gate, w_up):
+    mfma = _moe_on_matrix_cores(x, x.stride(0), D, w_gate, w_up)
+    _need(mfma or not frag, "moe_experts_gated: matrices in fragment order need bfloat16 rows "
+          "with 16-byte aligned starts")
+    if mfma:
         check(library("moe").kappai_moe_gemm_mfma(
             _ptr(x), _c_int(x.stride(0)), _ptr(w_gate), _ptr(w_up), _c_int(F), _c_int(D),
             _ptr(plan.tile_expert), _ptr(plan.pair_of_slot), _c_int(plan.top),
-            _c_int(plan.n_tiles), _ptr(out), _c_int(1), _stream()), "moe_gemm_mfma (gate, up)")
+            _c_int(plan.n_tiles), _ptr(out), _c_int(1), _c_int(_moe_few(plan)), _c_int(frag),
+            _stream()), "moe_gemm_mfma (gate, up)")
         return out
     check(library("moe").kappai_moe_gemm(
         _ptr(x), _c_int(x.stride(0)), _ptr(w_gate), _ptr(w_up), _c_int(F), _c_int(D),
@@ -1483,16 +1528,20 @@ def moe_experts_gated(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor,
 def moe_experts_down(act: torch.Tensor, w_down: torch.Tensor, plan: MoePlan) -> torch.Tensor:
     """``act W_down[e]^T`` for every slot of the plan: float32 [slots, D]."""
     _gpu("act", act, (F32, BF16))
-    _gpu("w_down", w_down, act.dtype)
     E, D, F = w_down.shape
+    w_down, frag = _moe_matrix(w_down)
+    _gpu("w_down", w_down, act.dtype)
     _need(tuple(act.shape) == (plan.n_tiles * plan.tile_rows, F),
-          lambda: f"moe_experts_down: act {tuple(act.shape)}, matrices {tuple(w_down.shape)}")
+          lambda: f"moe_experts_down: act {tuple(act.shape)}, matrices {(E, D, F)}")
     out = torch.empty((act.shape[0], D), dtype=F32, device=act.device)
-    if _moe_on_matrix_cores(act, F, F, w_down):
+    mfma = _moe_on_matrix_cores(act, F, F, w_down)
+    _need(mfma or not frag, "moe_experts_down: matrices in fragment order need bfloat16 rows")
+    if mfma:
         check(library("moe").kappai_moe_gemm_mfma(
             _ptr(act), _c_int(F), _ptr(w_down), _vp(0), _c_int(D), _c_int(F),
             _ptr(plan.tile_expert), _ptr(plan.pair_of_slot), _c_int(plan.top),
-            _c_int(plan.n_tiles), _ptr(out), _c_int(0), _stream()), "moe_gemm_mfma (down)")
+            _c_int(plan.n_tiles), _ptr(out), _c_int(0), _c_int(_moe_few(plan)), _c_int(frag),
+            _stream()), "moe_gemm_mfma (down)")
         return out
     check(library("moe").kappai_moe_gemm(
         _ptr(act), _c_int(F), _ptr(w_down), _vp(0), _c_int(D), _c_int(F),

@@ -12,7 +12,7 @@ from typing import Dict, List, Optional
 
 import torch
 
-from ..kernels import ops, profile
+from ..kernels import ops, profile, tuning
 from ..weights.spec import INIT_NORMAL, MATRIX, TensorSpec
 from .base import FeedForward, register_part
 
@@ -45,9 +45,17 @@ class MixtureOfExperts(FeedForward):
         self.router = tensors[self._router].to(torch.float32).contiguous()
 
         def stacked(key):
-            return torch.stack([tensors[names[key]].to(self.dtype) for names in self._expert]
-                               ).contiguous()
-        self.w_gate, self.w_up, self.w_down = stacked("gate"), stacked("up"), stacked("down")
+            w = torch.stack([tensors[names[key]].to(self.dtype) for names in self._expert]
+                            ).contiguous()
+            # bfloat16 matrices whose shape allows it are kept in the order the matrix-core
+            # kernel loads them, and only so
+            if w.is_cuda and tuning.FRAGMENT_ORDER and ops.ExpertFragments.fits(w):
+                return ops.ExpertFragments.of(w)
+            return w
+        up = stacked("up")
+        self.w_gate = stacked("gate")
+        self.w_up = up
+        self.w_down = stacked("down")
 
     def forward(self, x, batch):
         with profile.scope("router"):

@@ -159,12 +159,15 @@ def test_gelu_gate_alone_and_in_the_product(M):
 
 
 @pytest.mark.parametrize("dtype,tol", [(F32, 1e-5), (BF16, 2e-2)])
-@pytest.mark.parametrize("T,E,top,ff", [(1, 3, 1, 24), (7, 6, 3, 40), (200, 4, 4, 50),
-                                        (130, 17, 2, 96), (64, 70, 5, 16)])
-def test_mixture_of_experts(dtype, tol, T, E, top, ff):
+@pytest.mark.parametrize("T,E,top,ff,D", [(1, 3, 1, 24, 88), (7, 6, 3, 40, 88), (200, 4, 4, 50, 88),
+                                          (130, 17, 2, 96, 88), (64, 70, 5, 16, 88),
+                                          (300, 5, 2, 64, 96), (9, 8, 2, 48, 96),
+                                          (700, 3, 1, 160, 128)])
+def test_mixture_of_experts(dtype, tol, T, E, top, ff, D):
+    """(Widths of 96 and 128 with feed-forward widths of 64, 48 and 160: the bfloat16 matrices
+    lie in fragment order, all of them or the gate and up matrices only.)"""
     from kappai_amd.parts import MixtureOfExperts
     from kappai_amd.weights import random_tensors, stored_to_runtime
-    D = 88
     part = MixtureOfExperts("m.", D, ff, E, top, dtype, weight_suffix="")
     t = random_tensors(part.tensor_specs(), 5, std=0.15)
     t["m.router"] = (t["m.router"].float() * 6).to(BF16)       # no close calls between experts
