@@ -82,11 +82,12 @@ def _dapipel(width, mixers, heads, kv_heads, dim, vdim, window, ff, experts, top
 
 
 SHAPES.update({
-    # eight layers at a width of 1024: attention where the LFM2 pattern has it (2, 5, 7), a
-    # recurrent layer elsewhere; feed-forward 4608 dense or 16 experts of 2304, two a token
-    "dapipel-w1024": _dapipel(1024, "ggaggaga", 16, 8, 32, 64, 1024, 4608, 16, 2),
+    # eight layers at a width of 1024: attention where the LFM2 pattern has it (2, 5, 7; 16 heads
+    # on 4 kv heads, so each map's 16 heads share 4 kv heads as LFM2's 32 share 8), a recurrent
+    # layer elsewhere; feed-forward 4608 dense or 16 experts of 2304, two a token
+    "dapipel-w1024": _dapipel(1024, "ggaggaga", 16, 4, 32, 64, 1024, 4608, 16, 2),
     # the same at a width of 2048: heads of 128 values on maps of 64, feed-forward 8192
-    "dapipel-w2048": _dapipel(2048, "ggaggaga", 16, 8, 64, 128, 2048, 8192, 16, 2),
+    "dapipel-w2048": _dapipel(2048, "ggaggaga", 16, 4, 64, 128, 2048, 8192, 16, 2),
     # a tiny one for smoke runs
     "dapipel-tiny": _dapipel(64, "gaga", 4, 2, 8, 16, 24, 96, 4, 2, vocab=256, positions=512,
                              inner=48),
