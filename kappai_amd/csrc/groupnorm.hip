@@ -99,45 +99,6 @@ __global__ __launch_bounds__(GN_THREADS) void canon_conv_kernel(
   }
 }
 
-// The same for four neighbouring channels a thread (16-byte loads of h, 8- or 16-byte stores):
-// widths that are multiples of four.
-template <typename TO>
-__global__ __launch_bounds__(GN_THREADS) void canon_conv_vec_kernel(
-    const float* __restrict__ h, const float* __restrict__ taps, const float* __restrict__ state,
-    const int* __restrict__ row_pos, const int* __restrict__ row_seg,
-    const int* __restrict__ seg_start, const int* __restrict__ seg_slot, int n_taps, int D,
-    TO* __restrict__ out) {
-  const int t = blockIdx.x;
-  const int seg = row_seg[t], pos = row_pos[t];
-  const int local = t - seg_start[seg];
-  const float* st = state + (size_t)seg_slot[seg] * (n_taps - 1) * D;
-  for (int c = threadIdx.x * 4; c < D; c += GN_THREADS * 4) {
-    const float4 own = *reinterpret_cast<const float4*>(h + (size_t)t * D + c);
-    float acc[4] = {own.x, own.y, own.z, own.w};
-    for (int j = 0; j < n_taps; ++j) {
-      const int back = n_taps - 1 - j;
-      if (pos - back < 0) continue;
-      const float* src = (local - back >= 0) ? h + (size_t)(t - back) * D + c
-                                             : st + (size_t)(n_taps - 1 + local - back) * D + c;
-      const float4 v = *reinterpret_cast<const float4*>(src);
-      const float* tw = taps + (size_t)c * n_taps + j;
-      acc[0] = fmaf(tw[0], v.x, acc[0]);
-      acc[1] = fmaf(tw[n_taps], v.y, acc[1]);
-      acc[2] = fmaf(tw[2 * n_taps], v.z, acc[2]);
-      acc[3] = fmaf(tw[3 * n_taps], v.w, acc[3]);
-    }
-    TO* o = out + (size_t)t * D + c;
-    if (sizeof(TO) == 2) {
-      uint2 pk;
-      pk.x = pack_bf16x2(acc[0], acc[1]);
-      pk.y = pack_bf16x2(acc[2], acc[3]);
-      *reinterpret_cast<uint2*>(o) = pk;
-    } else {
-      *reinterpret_cast<float4*>(o) = make_float4(acc[0], acc[1], acc[2], acc[3]);
-    }
-  }
-}
-
 // The state after the step: the last n - 1 inputs of every segment's request, oldest first.  A
 // thread owns a channel of a segment and reads what it keeps of the old state before it writes.
 __global__ __launch_bounds__(GN_THREADS) void canon_state_kernel(
@@ -167,15 +128,7 @@ extern "C" int kappai_canon_conv(const float* h, const float* taps, float* state
                                  int out_is_bf16, hipStream_t stream) {
   if (T <= 0 || S <= 0) return 0;
   if (n_taps < 1 || n_taps > CANON_MAX_TAPS || S > 65535) return (int)hipErrorInvalidValue;
-  const bool vec = D % 4 == 0 && (uintptr_t)h % 16 == 0 && (uintptr_t)state % 16 == 0 &&
-                   (uintptr_t)out % 16 == 0;
-  if (out_is_bf16 && vec)
-    hipLaunchKernelGGL(canon_conv_vec_kernel<bf16_t>, dim3(T), dim3(GN_THREADS), 0, stream, h, taps,
-                       state, row_pos, row_seg, seg_start, seg_slot, n_taps, D, (bf16_t*)out);
-  else if (vec)
-    hipLaunchKernelGGL(canon_conv_vec_kernel<float>, dim3(T), dim3(GN_THREADS), 0, stream, h, taps,
-                       state, row_pos, row_seg, seg_start, seg_slot, n_taps, D, (float*)out);
-  else if (out_is_bf16)
+  if (out_is_bf16)
     hipLaunchKernelGGL(canon_conv_kernel<bf16_t>, dim3(T), dim3(GN_THREADS), 0, stream, h, taps,
                        state, row_pos, row_seg, seg_start, seg_slot, n_taps, D, (bf16_t*)out);
   else
