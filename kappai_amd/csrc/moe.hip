@@ -346,19 +346,23 @@ typedef __attribute__((ext_vector_type(4))) uint32_t moe_u32x4_t;
 // WF: the experts' matrices lie in fragment order (the host arranges them once): the 16 rows x
 // 32 of K that a matrix instruction takes are 1 KB in a row, lane after lane, tile (row tile,
 // step of K) after tile, so that a wave's load is one piece of memory instead of sixteen.
-template <int GATED, int NT, int U, bool WF>
+// BYROW: the block's four waves take four tiles in a row and the same columns (a step of many
+// rows: tiles in a row mostly belong to one expert, whose matrix the waves then read together,
+// once a block instead of once a tile); else they take one tile and four sets of columns.
+template <int GATED, int NT, int U, bool WF, bool BYROW>
 __global__ __launch_bounds__(MOE_MFMA_WAVES * WAVE) void moe_gemm_mfma_kernel(
     const bf16_t* __restrict__ a, int lda, const bf16_t* __restrict__ w0,
     const bf16_t* __restrict__ w1, int N, int K, const int* __restrict__ tile_expert,
-    const int* __restrict__ pair_of_slot, int top, void* __restrict__ out_v) {
+    const int* __restrict__ pair_of_slot, int top, int n_tiles, void* __restrict__ out_v) {
   constexpr int MT = MOE_TILE_M / 16;
   constexpr int NG = GATED ? 2 : 1;
-  const int tile = blockIdx.x;
+  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  const int tile = BYROW ? blockIdx.x * MOE_MFMA_WAVES + wave : blockIdx.x;
+  if (tile >= n_tiles) return;
   const int e = tile_expert[tile];
   if (e < 0) return;
-  const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
   const int col = lane % 16, kg = 8 * (lane / 16);
-  const int n0 = (blockIdx.y * MOE_MFMA_WAVES + wave) * 16 * NT;
+  const int n0 = BYROW ? blockIdx.y * 16 * NT : (blockIdx.y * MOE_MFMA_WAVES + wave) * 16 * NT;
   if (n0 >= N) return;
   const bf16_t* arow[MT];
   bool a_ok[MT];
@@ -462,17 +466,19 @@ extern "C" int kappai_moe_gemm_mfma(const void* a, int lda, const void* w0, cons
     return (int)hipErrorInvalidValue;
   if (w_frag && ((K % 32) || (N % 16))) return (int)hipErrorInvalidValue;
   const dim3 block(MOE_MFMA_WAVES * WAVE);
-#define MOE_MFMA_LAUNCH(G, NT_, U_)                                                              \
-  if (w_frag) MOE_MFMA_LAUNCH_WF(G, NT_, U_, true); else MOE_MFMA_LAUNCH_WF(G, NT_, U_, false)
-#define MOE_MFMA_LAUNCH_WF(G, NT_, U_, WF_)                                                      \
-  hipLaunchKernelGGL((moe_gemm_mfma_kernel<G, NT_, U_, WF_>),                                    \
-                     dim3(n_tiles, (N + 16 * NT_ * MOE_MFMA_WAVES - 1) / (16 * NT_ * MOE_MFMA_WAVES)), \
-                     block, 0, stream, (const bf16_t*)a, lda, (const bf16_t*)w0, (const bf16_t*)w1, \
-                     N, K, tile_expert, pair_of_slot, top, out)
+#define MOE_MFMA_LAUNCH(G, NT_, U_, BR_)                                                         \
+  if (w_frag) MOE_MFMA_LAUNCH_WF(G, NT_, U_, true, BR_); else MOE_MFMA_LAUNCH_WF(G, NT_, U_, false, BR_)
+#define MOE_MFMA_LAUNCH_WF(G, NT_, U_, WF_, BR_)                                                 \
+  hipLaunchKernelGGL(                                                                            \
+      (moe_gemm_mfma_kernel<G, NT_, U_, WF_, BR_>),                                              \
+      BR_ ? dim3((n_tiles + MOE_MFMA_WAVES - 1) / MOE_MFMA_WAVES, (N + 16 * NT_ - 1) / (16 * NT_)) \
+          : dim3(n_tiles, (N + 16 * NT_ * MOE_MFMA_WAVES - 1) / (16 * NT_ * MOE_MFMA_WAVES)),      \
+      block, 0, stream, (const bf16_t*)a, lda, (const bf16_t*)w0, (const bf16_t*)w1, N, K,         \
+      tile_expert, pair_of_slot, top, n_tiles, out)
   if (gated) {
-    if (few) { MOE_MFMA_LAUNCH(1, 1, 2); } else { MOE_MFMA_LAUNCH(1, 4, 1); }
+    if (few) { MOE_MFMA_LAUNCH(1, 1, 2, false); } else { MOE_MFMA_LAUNCH(1, 4, 1, true); }
   } else {
-    if (few) { MOE_MFMA_LAUNCH(0, 2, 2); } else { MOE_MFMA_LAUNCH(0, 4, 1); }
+    if (few) { MOE_MFMA_LAUNCH(0, 2, 2, false); } else { MOE_MFMA_LAUNCH(0, 4, 1, true); }
   }
 #undef MOE_MFMA_LAUNCH
 #undef MOE_MFMA_LAUNCH_WF
