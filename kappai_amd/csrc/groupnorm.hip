@@ -99,6 +99,58 @@ __global__ __launch_bounds__(GN_THREADS) void canon_conv_kernel(
   }
 }
 
+// The same for steps of many rows: a block takes CANON_ROWS rows in a row and a thread one
+// channel of them, with the inputs of the rows before in registers (a row's input is read once
+// and a bit, not once a tap).  A row near its segment's start takes what lies before the segment
+// from the state, as above.  MAXT: the most taps the instance takes; the sums run in the same
+// order as above.
+#define CANON_ROWS 8
+
+template <typename TO, int MAXT>
+__global__ __launch_bounds__(GN_THREADS) void canon_conv_rows_kernel(
+    const float* __restrict__ h, const float* __restrict__ taps, const float* __restrict__ state,
+    const int* __restrict__ row_pos, const int* __restrict__ row_seg,
+    const int* __restrict__ seg_start, const int* __restrict__ seg_slot, int n_taps, int D, int T,
+    TO* __restrict__ out) {
+  const int t0 = blockIdx.x * CANON_ROWS;
+  const int c = blockIdx.y * GN_THREADS + threadIdx.x;
+  if (c >= D) return;
+  float twb[MAXT];            // the tap for the input b rows back
+  float win[MAXT];            // win[b - 1]: the input b rows back in the batch (b = 1 ..)
+  float cur[CANON_ROWS];
+#pragma unroll
+  for (int b = 0; b < MAXT; ++b) {
+    twb[b] = b < n_taps ? taps[(size_t)c * n_taps + (n_taps - 1 - b)] : 0.f;
+    const int tr = t0 - 1 - b;
+    win[b] = (b < n_taps - 1 && tr >= 0) ? h[(size_t)tr * D + c] : 0.f;
+  }
+#pragma unroll
+  for (int r = 0; r < CANON_ROWS; ++r) cur[r] = t0 + r < T ? h[(size_t)(t0 + r) * D + c] : 0.f;
+#pragma unroll
+  for (int r = 0; r < CANON_ROWS; ++r) {
+    const int t = t0 + r;
+    if (t < T) {
+      const int seg = row_seg[t], pos = row_pos[t];
+      const int local = t - seg_start[seg];
+      float acc = cur[r];
+#pragma unroll
+      for (int b = MAXT - 1; b >= 1; --b) {
+        if (b <= n_taps - 1 && pos - b >= 0) {
+          const float v = local - b >= 0
+                              ? win[b - 1]
+                              : state[((size_t)seg_slot[seg] * (n_taps - 1) + (n_taps - 1 + local - b)) * D + c];
+          acc = fmaf(twb[b], v, acc);
+        }
+      }
+      acc = fmaf(twb[0], cur[r], acc);
+      from_f32(out + (size_t)t * D + c, acc);
+    }
+#pragma unroll
+    for (int b = MAXT - 1; b >= 1; --b) win[b] = win[b - 1];
+    win[0] = cur[r];
+  }
+}
+
 // The state after the step: the last n - 1 inputs of every segment's request, oldest first.  A
 // thread owns a channel of a segment and reads what it keeps of the old state before it writes.
 __global__ __launch_bounds__(GN_THREADS) void canon_state_kernel(
@@ -128,12 +180,24 @@ extern "C" int kappai_canon_conv(const float* h, const float* taps, float* state
                                  int out_is_bf16, hipStream_t stream) {
   if (T <= 0 || S <= 0) return 0;
   if (n_taps < 1 || n_taps > CANON_MAX_TAPS || S > 65535) return (int)hipErrorInvalidValue;
-  if (out_is_bf16)
+  const dim3 rows_grid((T + CANON_ROWS - 1) / CANON_ROWS, (D + GN_THREADS - 1) / GN_THREADS);
+#define CANON_ROWS_LAUNCH(TT, MAXT_)                                                             \
+  hipLaunchKernelGGL((canon_conv_rows_kernel<TT, MAXT_>), rows_grid, dim3(GN_THREADS), 0, stream,  \
+                     h, taps, state, row_pos, row_seg, seg_start, seg_slot, n_taps, D, T, (TT*)out)
+  if (T >= 8 * CANON_ROWS && rows_grid.y <= 65535) {
+    // many rows: a block a run of rows
+    if (out_is_bf16) {
+      if (n_taps <= 4) CANON_ROWS_LAUNCH(bf16_t, 4); else CANON_ROWS_LAUNCH(bf16_t, CANON_MAX_TAPS);
+    } else {
+      if (n_taps <= 4) CANON_ROWS_LAUNCH(float, 4); else CANON_ROWS_LAUNCH(float, CANON_MAX_TAPS);
+    }
+  } else if (out_is_bf16)
     hipLaunchKernelGGL(canon_conv_kernel<bf16_t>, dim3(T), dim3(GN_THREADS), 0, stream, h, taps,
                        state, row_pos, row_seg, seg_start, seg_slot, n_taps, D, (bf16_t*)out);
   else
     hipLaunchKernelGGL(canon_conv_kernel<float>, dim3(T), dim3(GN_THREADS), 0, stream, h, taps,
                        state, row_pos, row_seg, seg_start, seg_slot, n_taps, D, (float*)out);
+#undef CANON_ROWS_LAUNCH
   if (n_taps > 1)
     hipLaunchKernelGGL(canon_state_kernel, dim3((D + GN_THREADS - 1) / GN_THREADS, S),
                        dim3(GN_THREADS), 0, stream, h, state, seg_start, seg_slot, n_taps, D);

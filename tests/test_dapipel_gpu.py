@@ -76,16 +76,18 @@ def test_group_norm(width, groups):
 
 @pytest.mark.parametrize("taps", [1, 2, 4, 7])
 def test_input_convolution_over_portions_and_slots(taps):
-    """Two requests side by side in portions down to one row, a third that takes over a slot
-    whose state holds NaN from nobody: at position 0 the state must not be read."""
+    """Two requests side by side in portions down to one row and up to many, a third that takes
+    over a slot whose state holds NaN from nobody: at position 0 the state must not be read."""
     from kappai_amd.kernels import ops
-    D, n = (70 if taps == 2 else 72), [23, 31]      # (70: no 16-byte loads)
+    D, n = (70 if taps == 2 else 72), [23 + 45, 31 + 52]      # (70: no 16-byte loads)
     w = torch.randn(D, taps, generator=gen(6)) * 0.5
     h = [torch.randn(k, D, generator=gen(7 + i)) for i, k in enumerate(n)]
     want = [P.canon(x.double(), w) for x in h]
     state = torch.full((3, taps - 1, D), float("nan"), device=DEV)
     done, outs = [0, 0], [[], []]
-    for a, b in [(5, 1), (1, 2), (1, 1), (2, 9), (7, 1), (1, 1), (6, 16)]:
+    # (the last step has rows enough for the kernel that takes runs of eight rows a block: the
+    # second request starts in the middle of a run, both have their history in the state)
+    for a, b in [(5, 1), (1, 2), (1, 1), (2, 9), (7, 1), (1, 1), (6, 16), (45, 52)]:
         t = tables([(done[0], a), (done[1], b)], slots=[2, 0])
         rows = torch.cat([h[0][done[0]:done[0] + a], h[1][done[1]:done[1] + b]]).to(DEV)
         y = ops.canon_conv(rows, w.to(DEV), state, t["row_pos"], t["row_seg"], t["seg_start"],
