@@ -73,7 +73,11 @@ def test_named_shapes():
     assert named_shape("tiny-a") == TINY_A and named_shape("tiny-b") == TINY_B
     named_shape("tiny-a")["hidden_size"] = 1          # a copy: the table is not changed
     assert SHAPES["tiny-a"]["hidden_size"] == 64
-    with pytest.raises(KeyError, match="known: lfm2-1.2b"):
+    for name, layers in (("dapipel-w1024", 8), ("dapipel-w2048", 8), ("dapipel-tiny", 4)):
+        cfg = config_from_dict(named_shape(name))
+        assert cfg.architecture == "Dapipel" and len(cfg.layers) == layers
+    assert config_from_dict(named_shape("lfm2-like-w2048")).ff_dim == 8192
+    with pytest.raises(KeyError, match="known: .*lfm2-1.2b"):
         named_shape("lfm2-7b")
 
 
