@@ -431,3 +431,32 @@ def test_fused_decode_norm_and_convolution_equal_the_two_kernels(taps, groups):
         if step >= taps - 1:         # (before that the state's oldest places hold nothing yet)
             used = slots.long()
             assert torch.equal(states[0][used], states[1][used])
+
+
+def test_command_line(model_dirs, tmp_path):
+    """The command line on a model folder and in random-weights mode (a named shape), with the
+    sampling options of any other model; ``--time`` prints the stages of the new parts."""
+    import subprocess
+    import sys
+    from pathlib import Path
+    root = Path(__file__).resolve().parent.parent
+    prompt = [5, 17, 3, 88, 41, 7, 120]
+    cfg, t = P.read_model_dir(model_dirs["P"])
+    toks = list(prompt)
+    for _ in range(6):
+        toks.append(int(P.forward(cfg, t, toks)[-1].argmax()))
+    out = subprocess.run(
+        [sys.executable, "-m", "kappai_amd", "-m", str(model_dirs["P"]), "--dtype", "float32",
+         "-p", ",".join(map(str, prompt)), "-n", "6", "-t", "0", "--num-pages", "16", "--time"],
+        cwd=str(root), capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert [int(x) for x in out.stdout.split()] == toks[len(prompt):]
+    assert "scan" in out.stderr and "router" in out.stderr and "short_conv" in out.stderr
+    made = tmp_path / "made"
+    out = subprocess.run(
+        [sys.executable, str(root / "bin" / "kappai-cli"), "--random-weights", "dapipel-tiny",
+         "--model", str(made), "--weight-seed", "2", "--weight-std", "0.1", "-n", "5", "-t", "0.8",
+         "-k", "20", "-s", "3", "--num-pages", "16", "7 8 9 10"],
+        cwd=str(tmp_path), capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert len(out.stdout.split()) == 5 and (made / "config.json").is_file()
