@@ -24,7 +24,8 @@ def load_model(model_dir, dtype, device="cuda:0") -> Model:
     dtype = parse_dtype(dtype) if isinstance(dtype, str) else dtype
     config = load_config(model_dir)
     model = build_model(config, dtype)
-    tensors = check_and_load(Path(model_dir), model.tensor_specs(), dtype, device)
+    tensors = check_and_load(Path(model_dir), model.tensor_specs(), dtype, device,
+                             may_be_unused=getattr(model, "unused_tensor_names", ()))
     model.bind(tensors)
     return model
 

@@ -35,6 +35,8 @@ class Model:
         self.embedding, self.layers = embedding, list(layers)
         self.final_norm, self.head = final_norm, head
         self.embedding_position = embedding_position
+        # names a checkpoint may hold although this model reads none of them (a builder fills it)
+        self.unused_tensor_names: List[str] = []
         self.schedule: List[LayerCall] = list(schedule) if schedule is not None else [
             LayerCall(i) for i in range(len(self.layers))]
         self._check_schedule()

@@ -26,7 +26,7 @@ def build_dapipel(config: DapipelConfig, dtype: torch.dtype) -> Model:
         return make_part("norm", "group_rmsnorm", name=name, width=width, eps=config.norm_eps,
                          groups=config.norm_groups, dtype=dtype, suffix="")
 
-    layers = []
+    layers, unused = [], []
     for i, layer in enumerate(config.layers):
         p = f"l{i}."
         m = layer.mixer
@@ -50,6 +50,10 @@ def build_dapipel(config: DapipelConfig, dtype: torch.dtype) -> Model:
                                      hidden=layer.mlp["ff"], experts=layer.mlp["experts"],
                                      top=layer.mlp["top"], dtype=dtype, weight_suffix="")
         has_ff = feed_forward is not None
+        if not has_ff:
+            # a layer without feed-forward reads no second norm and no second convolution; a
+            # file that holds them all the same is no error
+            unused += [p + "norm2", p + "canon2"]
         layers.append(make_part(
             "block", "conv_input",
             mixer_norm=norm(p + "norm1"),
@@ -64,8 +68,10 @@ def build_dapipel(config: DapipelConfig, dtype: torch.dtype) -> Model:
                           max_positions=config.max_positions, width=width,
                           input_scale=config.embedding_scale)
     head = OutputHead("embed", config.vocab_size, width, tied_to=embedding, suffix="")
-    return Model(config, dtype, embedding, layers, norm("final.norm"), head,
-                 embedding_position=positions)
+    model = Model(config, dtype, embedding, layers, norm("final.norm"), head,
+                  embedding_position=positions)
+    model.unused_tensor_names = unused
+    return model
 
 
 register_architecture(ARCHITECTURE, DapipelConfig, build_dapipel)

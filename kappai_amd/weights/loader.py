@@ -77,8 +77,11 @@ def _weight_files(model_dir: Path) -> List[Path]:
 
 
 def check_and_load(model_dir, specs: Iterable[TensorSpec], compute_dtype: torch.dtype,
-                   device) -> Dict[str, torch.Tensor]:
-    """Check the file(s) against ``specs`` and return ``{name: tensor on device}``."""
+                   device, may_be_unused: Iterable[str] = ()) -> Dict[str, torch.Tensor]:
+    """Check the file(s) against ``specs`` and return ``{name: tensor on device}``.
+    ``may_be_unused``: names that a file may hold although the model built from its config.json
+    reads none of them (tensors of a sublayer that the configuration switches off); they are
+    neither loaded nor reported."""
     model_dir = Path(model_dir)
     specs = {s.name: s for s in specs}
     files = []
@@ -93,7 +96,8 @@ def check_and_load(model_dir, specs: Iterable[TensorSpec], compute_dtype: torch.
             for n in f.names():
                 where[n] = f
         missing = sorted(n for n in specs if n not in where)
-        unexpected = sorted(n for n in where if n not in specs)
+        tolerated = set(may_be_unused)
+        unexpected = sorted(n for n in where if n not in specs and n not in tolerated)
         wrong = []
         for n, s in specs.items():
             if n in where:

@@ -130,3 +130,27 @@ def test_schedules_float32(monkeypatch, tmp_path, model_dirs, name, family):
     got = run_emulated(monkeypatch, model_dirs[name], steps, index, peak, tmp_path)
     assert len(got) == sum(len(t) for t in requests.values())
     assert_matches_plain(got, model_dirs[name], requests, "float32", (name, family))
+
+
+def test_a_file_may_hold_the_norm_and_convolution_of_a_feed_forward_that_is_switched_off(
+        tmp_path, model_dirs):
+    """Layer 2 of configuration P has no feed-forward.  A checkpoint that holds ``l2.norm2`` and
+    ``l2.canon2`` all the same loads (they are not read); any other stray tensor is an error."""
+    from kappai_amd.weights import WeightsError
+    from kappai_amd.weights.safetensors_io import SafetensorsFile, write_safetensors
+    import shutil
+    f = SafetensorsFile(model_dirs["P"] / "model.safetensors")
+    tensors = {n: f.read(n) for n in f.names()}
+    f.close()
+    tensors["l2.norm2"] = torch.ones(96, dtype=torch.bfloat16)
+    tensors["l2.canon2"] = torch.zeros(96, 3, dtype=torch.bfloat16)
+    folder = tmp_path / "more"
+    folder.mkdir()
+    shutil.copy(model_dirs["P"] / "config.json", folder / "config.json")
+    write_safetensors(folder / "model.safetensors", tensors)
+    model = load_model(folder, "float32", device="cpu")
+    assert model.bound
+    tensors["l1.norm3"] = torch.ones(96, dtype=torch.bfloat16)
+    write_safetensors(folder / "model.safetensors", tensors)
+    with pytest.raises(WeightsError, match="unexpected tensors .1.: l1.norm3"):
+        load_model(folder, "float32", device="cpu")

@@ -49,10 +49,10 @@ INIT_P = dict(seed=11, std=0.08, norm_jitter=0.1)
 
 # one group (the plain RMS norm), one tap (the convolution keeps no history), six heads on one kv
 # head, a window of one key (a position sees itself only) beside one of 33, one expert a token
-TINY_Q = config(200, 64, 300, 0.5, 1e-6, 1, 1, [
+TINY_Q = config(200, 64, 300, 0.75, 1e-6, 1, 1, [
     attention(6, 1, 8, 8, 1, 0.35, 0.5, moe(24, 3, 1)),
     mingru(48, None),
-    attention(2, 2, 32, 64, 33, 0.18, 0.7, dense(96)),
+    attention(2, 2, 24, 48, 33, 0.18, 0.7, dense(96)),
 ])
 INIT_Q = dict(seed=12, std=0.1, norm_jitter=0.05)
 
@@ -65,7 +65,7 @@ INIT_R = dict(seed=13, std=0.07, norm_jitter=0.1)
 
 # attention only, heads of 80 (values) on maps of 40, a window that is no multiple of a page
 TINY_S = config(150, 56, 512, 2.0, 1e-5, 2, 2, [
-    attention(2, 1, 40, 80, 37, 0.16, 0.6, dense(48)),
+    attention(2, 1, 40, 80, 37, 0.16, 0.65, dense(48)),
     attention(1, 1, 16, 16, 50, 0.25, 0.3, moe(32, 5, 2)),
 ])
 INIT_S = dict(seed=14, std=0.1, norm_jitter=0.1)
