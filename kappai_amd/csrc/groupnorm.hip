@@ -269,6 +269,87 @@ __global__ __launch_bounds__(GN_STEP_THREADS) void add_group_rmsnorm_canon_step_
   }
 }
 
+// The same with everything a thread needs asked for at once: the residual and its update, and
+// for the same columns the norm's weight, the taps and the state, so that the kernel makes one
+// trip to memory before the sums and none after.  Widths up to GN_STEP_MAXC * 1024 columns and up
+// to MAXT taps.
+#define GN_STEP_MAXC 4
+
+template <typename TO, int MAXT>
+__global__ __launch_bounds__(GN_STEP_THREADS) void add_group_rmsnorm_canon_step_early_kernel(
+    float* __restrict__ resid, const void* __restrict__ delta, int delta_kind, int n_part,
+    size_t part_stride, const float* __restrict__ w, float eps, int groups, int D,
+    const float* __restrict__ taps, float* __restrict__ state, const int* __restrict__ row_pos,
+    const int* __restrict__ seg_slot, int n_taps, TO* __restrict__ out) {
+  extern __shared__ float row[];
+  float* scale = row + D;
+  const int r = blockIdx.x;
+  float* x = resid + (size_t)r * D;
+  const int pos = row_pos[r];
+  float* st = state + (size_t)seg_slot[r] * (n_taps - 1) * D;
+  float xv[GN_STEP_MAXC], wv[GN_STEP_MAXC], keep[GN_STEP_MAXC][MAXT], tw[GN_STEP_MAXC][MAXT];
+#pragma unroll
+  for (int q = 0; q < GN_STEP_MAXC; ++q) {
+    const int c = threadIdx.x + q * GN_STEP_THREADS;
+    if (c < D) {
+      float v = x[c];
+      if (delta_kind == 1) {
+        v += bf16_to_f32(((const bf16_t*)delta)[(size_t)r * D + c]);
+      } else if (delta_kind == 2) {
+        const float* p = (const float*)delta + (size_t)r * D + c;
+        for (int s = 0; s < n_part; ++s) v += p[s * part_stride];
+      }
+      xv[q] = v;
+      wv[q] = w[c];
+#pragma unroll
+      for (int k = 0; k < MAXT; ++k) {
+        tw[q][k] = k < n_taps ? taps[(size_t)c * n_taps + k] : 0.f;
+        keep[q][k] = (k < n_taps - 1 && pos - (n_taps - 1 - k) >= 0) ? st[(size_t)k * D + c] : 0.f;
+      }
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < GN_STEP_MAXC; ++q) {
+    const int c = threadIdx.x + q * GN_STEP_THREADS;
+    if (c < D) {
+      row[c] = xv[q];
+      if (delta_kind) x[c] = xv[q];
+    }
+  }
+  __syncthreads();
+  const int gs = D / groups;
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  for (int g = wave; g < groups; g += GN_STEP_THREADS / WAVE) {
+    float ss = 0.f;
+    for (int i = lane; i < gs; i += WAVE) {
+      const float v = row[g * gs + i];
+      ss = fmaf(v, v, ss);
+    }
+    ss = wave_sum(ss);
+    if (lane == 0) scale[g] = 1.0f / sqrtf(ss / (float)gs + eps);
+  }
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < GN_STEP_MAXC; ++q) {
+    const int c = threadIdx.x + q * GN_STEP_THREADS;
+    if (c < D) {
+      const float h = xv[q] * scale[c / gs] * wv[q];
+      float acc = h;
+#pragma unroll
+      for (int k = 0; k < MAXT; ++k) {
+        if (k < n_taps - 1) {
+          acc = fmaf(tw[q][k], keep[q][k], acc);
+          if (k > 0) st[(size_t)(k - 1) * D + c] = keep[q][k];
+        } else if (k == n_taps - 1) {
+          acc = fmaf(tw[q][k], h, acc);
+        }
+      }
+      if (n_taps > 1) st[(size_t)(n_taps - 2) * D + c] = h;
+      from_f32(out + (size_t)r * D + c, acc);
+    }
+  }
+}
+
 extern "C" int kappai_add_group_rmsnorm_canon_step(float* resid, const void* delta, int delta_kind,
                                                    int n_part, int T, int D, const float* w,
                                                    float eps, int groups, const float* taps,
@@ -282,6 +363,17 @@ extern "C" int kappai_add_group_rmsnorm_canon_step(float* resid, const void* del
   const size_t lds = (size_t)(D + groups) * sizeof(float);
   if (lds > 64 * 1024) return (int)hipErrorInvalidValue;
   const size_t ps = (size_t)T * D;
+  if (D <= GN_STEP_MAXC * GN_STEP_THREADS && n_taps <= 4) {
+    if (out_is_bf16)
+      hipLaunchKernelGGL((add_group_rmsnorm_canon_step_early_kernel<bf16_t, 4>), dim3(T),
+                         dim3(GN_STEP_THREADS), lds, stream, resid, delta, delta_kind, n_part, ps, w,
+                         eps, groups, D, taps, state, row_pos, seg_slot, n_taps, (bf16_t*)out);
+    else
+      hipLaunchKernelGGL((add_group_rmsnorm_canon_step_early_kernel<float, 4>), dim3(T),
+                         dim3(GN_STEP_THREADS), lds, stream, resid, delta, delta_kind, n_part, ps, w,
+                         eps, groups, D, taps, state, row_pos, seg_slot, n_taps, (float*)out);
+    KAPPAI_RETURN_LAUNCH_STATUS();
+  }
   if (out_is_bf16)
     hipLaunchKernelGGL(add_group_rmsnorm_canon_step_kernel<bf16_t>, dim3(T), dim3(GN_STEP_THREADS), lds,
                        stream, resid, delta, delta_kind, n_part, ps, w, eps, groups, D, taps, state,

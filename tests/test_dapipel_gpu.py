@@ -293,8 +293,9 @@ def test_differential_attention_finds_one_key(dtype, tol, window):
 # ---------------------------------------------------------------------------------------------
 # whole models
 # ---------------------------------------------------------------------------------------------
-LENGTHS = {"P": [70, 45, 100, 37], "Q": [66, 35, 90], "R": [50, 81, 36], "S": [97, 40, 71]}
-MIXED_LENGTHS = {"P": [70, 45, 100, 37, 83, 64, 29, 58], "Q": [66, 35, 90, 41, 23, 77, 50, 64, 81],
+LENGTHS = {"P": [70, 45, 100, 37], "Q": [66, 35, 90], "R": [50, 81, 36], "S": [97, 40, 71],
+           "T": [80, 33, 101]}
+MIXED_LENGTHS = {"T": [61, 48, 97, 35, 80, 66, 27, 59], "P": [70, 45, 100, 37, 83, 64, 29, 58], "Q": [66, 35, 90, 41, 23, 77, 50, 64, 81],
                  "R": [50, 81, 36, 67, 44, 72, 90], "S": [66, 40, 85, 37, 58, 49, 92]}
 
 
@@ -334,7 +335,7 @@ def replay(model_dir, dtype, steps, index, max_tokens, out_dir, slots=4, graphs=
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "T"])
 @pytest.mark.parametrize("family", ["whole", "prefill_then_decode", "changing_portions", "mixed"])
 def test_schedules(tmp_path, model_dirs, name, family, dtype):
     """Every logit of every request.  The mixed family runs in a pool smaller than its requests
@@ -353,17 +354,17 @@ def test_schedules(tmp_path, model_dirs, name, family, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_past_every_window(tmp_path, model_dirs, dtype):
-    """A short prompt and 330 tokens one by one (windows of 20 and 37 passed many times, pages
+    """A short prompt and 330 tokens one by one (windows of 19, 20 and 41 passed many times, pages
     given back and taken again, the block tables of a graph grown), two requests side by side."""
-    for name in ("P", "S"):
+    for name in ("P", "T"):
         requests = make_requests(TINY[name][0]["vocab"], [350, 290], seed=22)
         plans = {"r0": (0, [20] + [1] * 330), "r1": (5, [3] + [1] * 287)}
         steps, index, peak = schedules.build(requests, plans)
         got, runner = replay(model_dirs[name], dtype, steps, index, peak, tmp_path / name)
         # (in bfloat16 the model with experts meets a close call early; its 32-bit run and the
-        # model without close calls among its first hundreds of rows carry the comparison)
+        # model without experts carry the comparison)
         assert_matches_plain(got, model_dirs[name], requests, dtype, (name, dtype),
-                             min_strict=0.3 if name == "S" else 0.0)
+                             min_strict=1.0 if name == "T" else 0.0)
         assert runner.graph_replays > 250
 
 
@@ -407,7 +408,7 @@ def test_greedy_generation_through_the_engine(model_dirs):
         eng.shutdown()
 
 
-@pytest.mark.parametrize("taps,groups", [(4, 3), (1, 1), (2, 8)])
+@pytest.mark.parametrize("taps,groups", [(4, 3), (1, 1), (2, 8), (7, 2)])
 def test_fused_decode_norm_and_convolution_equal_the_two_kernels(taps, groups):
     """The one kernel of a decode step (residual sum, grouped norm, convolution, state shift)
     against the norm kernel followed by the convolution's two, over several steps of three rows in

@@ -70,7 +70,16 @@ TINY_S = config(150, 56, 512, 2.0, 1e-5, 2, 2, [
 ])
 INIT_S = dict(seed=14, std=0.1, norm_jitter=0.1)
 
-TINY = {"P": (TINY_P, INIT_P), "Q": (TINY_Q, INIT_Q), "R": (TINY_R, INIT_R),
+# no experts (no router whose choice rounding could change): attention with two windows around a
+# recurrent layer, five groups
+TINY_T = config(180, 80, 512, 1.3, 1e-5, 5, 3, [
+    attention(4, 2, 16, 32, 19, 0.25, 0.35, dense(64)),
+    mingru(64, dense(48)),
+    attention(2, 2, 24, 16, 41, 0.2, 0.55, None),
+])
+INIT_T = dict(seed=15, std=0.1, norm_jitter=0.1)
+
+TINY = {"T": (TINY_T, INIT_T), "P": (TINY_P, INIT_P), "Q": (TINY_Q, INIT_Q), "R": (TINY_R, INIT_R),
         "S": (TINY_S, INIT_S)}
 
 
