@@ -14,6 +14,7 @@
 // [page][kv_head][head_dim][page_size], which is what the matrix-core kernels want.  Token p of
 // a request lives in page block_table[p / page_size] at offset p % page_size.
 #include "common.h"
+#include "score_mods.h"
 
 #define MAX_HEAD_DIM 512
 
@@ -303,13 +304,13 @@ __device__ __forceinline__ float dot_row(const float* __restrict__ qs,
 
 #define ATT_NPL (MAX_HEAD_DIM / WAVE)
 
-template <typename T>
+template <typename T, bool MODS>
 __global__ __launch_bounds__(64) void paged_attention_rows_kernel(
     const T* __restrict__ q, int q_stride, const T* __restrict__ k_pool,
     const T* __restrict__ v_pool, T* __restrict__ out, int out_stride,
     const int* __restrict__ row_pos, const int* __restrict__ row_seg,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int d, int ps, int window,
-    float scale) {
+    float scale, kappai_score_mods mods) {
   __shared__ float qs[MAX_HEAD_DIM];
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const int g = h / (H / G);
@@ -333,6 +334,7 @@ __global__ __launch_bounds__(64) void paged_attention_rows_kernel(
     if (valid) {
       const size_t pg = (size_t)bt[tk / ps] * G + g;
       s = dot_row(qs, k_pool + (pg * ps + tk % ps) * d, d) * scale;
+      if (MODS) s = kappai_modified_score(mods, s, h, pos - tk);
       voff = (unsigned long long)(pg * d * ps + tk % ps);
     }
     const float m_new = fmaxf(m, wave_max(s));
@@ -355,6 +357,7 @@ __global__ __launch_bounds__(64) void paged_attention_rows_kernel(
     }
     m = m_new;
   }
+  if (MODS && mods.sink != nullptr) l += expf(mods.sink[h] - m);
   const float inv = 1.0f / l;
   T* o = out + (size_t)t * out_stride + (size_t)h * d;
 #pragma unroll
@@ -364,24 +367,47 @@ __global__ __launch_bounds__(64) void paged_attention_rows_kernel(
   }
 }
 
+template <typename T, bool MODS>
+static void rows_launch(const void* q, int q_stride, const void* k_pool, const void* v_pool,
+                        void* out, int out_stride, const int* row_pos, const int* row_seg,
+                        const int* block_tables, int max_blocks, int T_, int H, int G, int d,
+                        int ps, int window, float scale, kappai_score_mods mods,
+                        hipStream_t stream) {
+  hipLaunchKernelGGL((paged_attention_rows_kernel<T, MODS>), dim3(T_, H), dim3(WAVE), 0, stream,
+                     (const T*)q, q_stride, (const T*)k_pool, (const T*)v_pool, (T*)out,
+                     out_stride, row_pos, row_seg, block_tables, max_blocks, H, G, d, ps, window,
+                     scale, mods);
+}
+
+// `mods` (may be null): see score_mods.h
+extern "C" int kappai_paged_attention_rows_scored(
+    const void* q, int q_stride, const void* k_pool, const void* v_pool, void* out,
+    int out_stride, const int* row_pos, const int* row_seg, const int* block_tables,
+    int max_blocks, int T, int H, int G, int d, int ps, int window, float scale, int is_bf16,
+    const kappai_score_mods* mods, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (d > MAX_HEAD_DIM || d % 8 || G < 1 || H % G || H > 65535) return (int)hipErrorInvalidValue;
+  const bool on = mods != nullptr && (mods->softcap > 0.f || mods->dist_bias || mods->sink);
+  if (on && mods->dist_bias && mods->dist_cols < 1) return (int)hipErrorInvalidValue;
+  const kappai_score_mods m = on ? *mods : kappai_score_mods{0.f, nullptr, 0, nullptr};
+#define ROWS_ARGS q, q_stride, k_pool, v_pool, out, out_stride, row_pos, row_seg, block_tables, \
+                  max_blocks, T, H, G, d, ps, window, scale, m, stream
+  if (is_bf16) {
+    if (on) rows_launch<bf16_t, true>(ROWS_ARGS); else rows_launch<bf16_t, false>(ROWS_ARGS);
+  } else {
+    if (on) rows_launch<float, true>(ROWS_ARGS); else rows_launch<float, false>(ROWS_ARGS);
+  }
+#undef ROWS_ARGS
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
 extern "C" int kappai_paged_attention_rows(const void* q, int q_stride, const void* k_pool,
                                            const void* v_pool, void* out, int out_stride,
                                            const int* row_pos, const int* row_seg,
                                            const int* block_tables, int max_blocks, int T, int H,
                                            int G, int d, int ps, int window, float scale,
                                            int is_bf16, hipStream_t stream) {
-  if (T <= 0) return 0;
-  if (d > MAX_HEAD_DIM || d % 8 || G < 1 || H % G || H > 65535) return (int)hipErrorInvalidValue;
-  dim3 grid(T, H);
-  if (is_bf16)
-    hipLaunchKernelGGL(paged_attention_rows_kernel<bf16_t>, grid, dim3(WAVE), 0, stream,
-                       (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)v_pool,
-                       (bf16_t*)out, out_stride, row_pos, row_seg, block_tables, max_blocks, H, G,
-                       d, ps, window, scale);
-  else
-    hipLaunchKernelGGL(paged_attention_rows_kernel<float>, grid, dim3(WAVE), 0, stream,
-                       (const float*)q, q_stride, (const float*)k_pool, (const float*)v_pool,
-                       (float*)out, out_stride, row_pos, row_seg, block_tables, max_blocks, H, G, d,
-                       ps, window, scale);
-  KAPPAI_RETURN_LAUNCH_STATUS();
+  return kappai_paged_attention_rows_scored(q, q_stride, k_pool, v_pool, out, out_stride, row_pos,
+                                            row_seg, block_tables, max_blocks, T, H, G, d, ps,
+                                            window, scale, is_bf16, nullptr, stream);
 }

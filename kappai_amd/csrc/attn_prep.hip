@@ -1,0 +1,241 @@
+// What stands between an attention layer's projections and the paged attention kernels when the
+// layer is not the plain grouped-query form: queries, keys and values are normalised, scaled,
+// rotated and laid out as heads of one size D (zeros behind what a head really holds), keys go to
+// the key pool [page][kv_head][slot][D], values transposed to [page][kv_head][D][slot].
+//
+//   projection_norm_store   RMS norm over the WHOLE q projection (all heads at once) and over the
+//                           whole k projection, a query factor that grows with the position,
+//                           heads of d (q, k) and dv (v) widened to D
+//   latent_store            keys and values from one latent vector a token: the normalised latent
+//                           c [r] and a rotated part [rot] shared by all heads become the one kv
+//                           head's key [c | rot | 0]; c again is its value; the queries' rotated
+//                           parts are rotated and put behind the r places that the product with
+//                           the keys' up-projection fills (headwise_linear)
+//   headwise_linear         y[t, h, :] = W[h] x[t, h, :], a matrix per head
+#include "common.h"
+
+#define AP_THREADS 256
+
+// ---------------------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(AP_THREADS) void projection_norm_store_kernel(
+    const T* __restrict__ proj, int stride, const float* __restrict__ q_norm_w,
+    const float* __restrict__ k_norm_w, float eps, float temp_coef, int temp_every,
+    T* __restrict__ k_pool, T* __restrict__ v_pool, const int* __restrict__ row_pos,
+    const int* __restrict__ row_seg, const int* __restrict__ block_tables, int max_blocks, int H,
+    int G, int d, int dv, int D, int ps, T* __restrict__ q_out) {
+  __shared__ float red[16];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int pos = row_pos[t];
+  const T* row = proj + (size_t)t * stride;
+  const int nq = H * d, nk = G * d;
+  float fq = 1.f, fk = 1.f;
+  if (q_norm_w != nullptr) {
+    float ss = 0.f;
+    for (int e = tid; e < nq; e += AP_THREADS) { const float v = to_f32(row[e]); ss = fmaf(v, v, ss); }
+    fq = 1.0f / sqrtf(block_sum(ss, red) / (float)nq + eps);
+  }
+  if (k_norm_w != nullptr) {
+    float ss = 0.f;
+    for (int e = tid; e < nk; e += AP_THREADS) {
+      const float v = to_f32(row[nq + e]);
+      ss = fmaf(v, v, ss);
+    }
+    fk = 1.0f / sqrtf(block_sum(ss, red) / (float)nk + eps);
+  }
+  if (temp_coef != 0.f) fq *= 1.0f + temp_coef * logf((float)((pos + 1) / temp_every + 1));
+  for (int i = tid; i < H * D; i += AP_THREADS) {
+    const int h = i / D, e = i % D;
+    float v = 0.f;
+    if (e < d) v = to_f32(row[h * d + e]) * fq * (q_norm_w ? q_norm_w[h * d + e] : 1.f);
+    from_f32(q_out + (size_t)t * H * D + i, v);
+  }
+  if (k_pool == nullptr) return;
+  const size_t page = (size_t)block_tables[(size_t)row_seg[t] * max_blocks + pos / ps];
+  const int slot = pos % ps;
+  for (int i = tid; i < G * D; i += AP_THREADS) {
+    const int g = i / D, e = i % D;
+    float kv = 0.f, vv = 0.f;
+    if (e < d) kv = to_f32(row[nq + g * d + e]) * fk * (k_norm_w ? k_norm_w[g * d + e] : 1.f);
+    if (e < dv) vv = to_f32(row[nq + nk + g * dv + e]);
+    from_f32(k_pool + ((page * G + g) * ps + slot) * D + e, kv);
+    from_f32(v_pool + ((page * G + g) * D + e) * ps + slot, vv);
+  }
+}
+
+extern "C" int kappai_projection_norm_store(
+    const void* proj, int stride, const float* q_norm_w, const float* k_norm_w, float eps,
+    float temp_coef, int temp_every, void* k_pool, void* v_pool, const int* row_pos,
+    const int* row_seg, const int* block_tables, int max_blocks, int T, int H, int G, int d,
+    int dv, int D, int ps, void* q_out, int is_bf16, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H < 1 || G < 1 || d < 1 || dv < 1 || D < d || D < dv || ps < 1 || temp_every < 1)
+    return (int)hipErrorInvalidValue;
+  if (is_bf16)
+    hipLaunchKernelGGL(projection_norm_store_kernel<bf16_t>, dim3(T), dim3(AP_THREADS), 0, stream,
+                       (const bf16_t*)proj, stride, q_norm_w, k_norm_w, eps, temp_coef, temp_every,
+                       (bf16_t*)k_pool, (bf16_t*)v_pool, row_pos, row_seg, block_tables,
+                       max_blocks, H, G, d, dv, D, ps, (bf16_t*)q_out);
+  else
+    hipLaunchKernelGGL(projection_norm_store_kernel<float>, dim3(T), dim3(AP_THREADS), 0, stream,
+                       (const float*)proj, stride, q_norm_w, k_norm_w, eps, temp_coef, temp_every,
+                       (float*)k_pool, (float*)v_pool, row_pos, row_seg, block_tables, max_blocks,
+                       H, G, d, dv, D, ps, (float*)q_out);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
+// rot_mode 1: pairs (j, j + rot_dims / 2); 2: pairs (2j, 2j + 1).  cos / sin [positions,
+// rot_dims / 2].  Only the first rot_dims of the rot places turn; the rest pass as they are.
+__device__ __forceinline__ float rotated(const float* x, int e, int rot_dims, int rot_mode,
+                                         const float* ct, const float* st) {
+  if (e >= rot_dims || rot_mode == 0) return x[e];
+  const int half = rot_dims / 2;
+  int j, partner;
+  bool first;
+  if (rot_mode == 1) { first = e < half; j = first ? e : e - half; partner = first ? e + half : e - half; }
+  else { first = (e & 1) == 0; j = e / 2; partner = e ^ 1; }
+  const float c = ct[j], s = st[j];
+  return first ? x[e] * c - x[partner] * s : x[e] * c + x[partner] * s;
+}
+
+template <typename T>
+__global__ __launch_bounds__(AP_THREADS) void latent_store_kernel(
+    const T* __restrict__ q, int q_stride, const T* __restrict__ kv, int kv_stride,
+    const float* __restrict__ c_norm_w, float eps, const float* __restrict__ cos_tab,
+    const float* __restrict__ sin_tab, int rot_dims, int rot_mode, T* __restrict__ k_pool,
+    T* __restrict__ v_pool, const int* __restrict__ row_pos, const int* __restrict__ row_seg,
+    const int* __restrict__ block_tables, int max_blocks, int H, int d, int rot, int r, int D,
+    int ps, T* __restrict__ q_out) {
+  extern __shared__ float sh[];            // (H + 1) * rot floats: the parts that turn
+  __shared__ float red[16];
+  const int t = blockIdx.x, tid = threadIdx.x;
+  const int pos = row_pos[t];
+  const T* kvr = kv + (size_t)t * kv_stride;
+  const T* qr = q + (size_t)t * q_stride;
+  const float* ct = cos_tab + (size_t)pos * (rot_dims / 2);
+  const float* st = sin_tab + (size_t)pos * (rot_dims / 2);
+  float ss = 0.f;
+  for (int e = tid; e < r; e += AP_THREADS) { const float v = to_f32(kvr[e]); ss = fmaf(v, v, ss); }
+  for (int i = tid; i < (H + 1) * rot; i += AP_THREADS) {
+    const int h = i / rot, e = i % rot;
+    sh[i] = h < H ? to_f32(qr[h * (d + rot) + d + e]) : to_f32(kvr[r + e]);
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)r + eps);      // (barrier inside)
+  for (int i = tid; i < H * (D - r); i += AP_THREADS) {
+    const int h = i / (D - r), e = i % (D - r);
+    const float v = e < rot ? rotated(sh + h * rot, e, rot_dims, rot_mode, ct, st) : 0.f;
+    from_f32(q_out + (size_t)t * H * D + (size_t)h * D + r + e, v);
+  }
+  if (k_pool == nullptr) return;
+  const size_t page = (size_t)block_tables[(size_t)row_seg[t] * max_blocks + pos / ps];
+  const int slot = pos % ps;
+  for (int e = tid; e < D; e += AP_THREADS) {
+    float kvv = 0.f, vv = 0.f;
+    if (e < r) kvv = vv = to_f32(kvr[e]) * inv * c_norm_w[e];
+    else if (e < r + rot) kvv = rotated(sh + H * rot, e - r, rot_dims, rot_mode, ct, st);
+    from_f32(k_pool + (page * ps + slot) * D + e, kvv);
+    from_f32(v_pool + (page * D + e) * ps + slot, vv);
+  }
+}
+
+extern "C" int kappai_latent_store(const void* q, int q_stride, const void* kv, int kv_stride,
+                                   const float* c_norm_w, float eps, const float* cos_tab,
+                                   const float* sin_tab, int rot_dims, int rot_mode, void* k_pool,
+                                   void* v_pool, const int* row_pos, const int* row_seg,
+                                   const int* block_tables, int max_blocks, int T, int H, int d,
+                                   int rot, int r, int D, int ps, void* q_out, int is_bf16,
+                                   hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (H < 1 || d < 1 || rot < 0 || r < 1 || D < r + rot || rot_dims > rot || rot_dims % 2 ||
+      rot_mode < 0 || rot_mode > 2 || (rot_mode && rot_dims && (!cos_tab || !sin_tab)))
+    return (int)hipErrorInvalidValue;
+  const size_t lds = (size_t)(H + 1) * (rot > 0 ? rot : 1) * sizeof(float);
+  if (lds > 48 * 1024) return (int)hipErrorInvalidValue;
+  if (is_bf16)
+    hipLaunchKernelGGL(latent_store_kernel<bf16_t>, dim3(T), dim3(AP_THREADS), lds, stream,
+                       (const bf16_t*)q, q_stride, (const bf16_t*)kv, kv_stride, c_norm_w, eps,
+                       cos_tab, sin_tab, rot_dims, rot_mode, (bf16_t*)k_pool, (bf16_t*)v_pool,
+                       row_pos, row_seg, block_tables, max_blocks, H, d, rot, r, D, ps,
+                       (bf16_t*)q_out);
+  else
+    hipLaunchKernelGGL(latent_store_kernel<float>, dim3(T), dim3(AP_THREADS), lds, stream,
+                       (const float*)q, q_stride, (const float*)kv, kv_stride, c_norm_w, eps,
+                       cos_tab, sin_tab, rot_dims, rot_mode, (float*)k_pool, (float*)v_pool,
+                       row_pos, row_seg, block_tables, max_blocks, H, d, rot, r, D, ps,
+                       (float*)q_out);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
+// y[t, h, o] = sum_i W[h, o, i] x[t, h, i]: W [H, n_out, n_in] in the activations' dtype, x and y
+// with a row stride and a head stride each, float accumulation.  A block takes 32 rows x 64
+// outputs of one head; x and W tiles go through LDS in steps of 32 along i.
+// ---------------------------------------------------------------------------------------
+#define HW_BM 32
+#define HW_BN 64
+#define HW_BK 32
+
+template <typename T>
+__global__ __launch_bounds__(256) void headwise_linear_kernel(
+    const T* __restrict__ x, int x_row, int x_head, const T* __restrict__ w, int n_out, int n_in,
+    T* __restrict__ y, int y_row, int y_head, int rows) {
+  __shared__ float xs[HW_BM][HW_BK + 1];
+  __shared__ float ws[HW_BN][HW_BK + 1];
+  const int h = blockIdx.z, m0 = blockIdx.x * HW_BM, n0 = blockIdx.y * HW_BN;
+  const int tid = threadIdx.x;
+  const int tx = tid % 16, ty = tid / 16;          // outputs 4 tx .. 4 tx + 3, rows 2 ty, 2 ty + 1
+  const T* wh = w + (size_t)h * n_out * n_in;
+  float acc[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  for (int k0 = 0; k0 < n_in; k0 += HW_BK) {
+    for (int i = tid; i < HW_BM * HW_BK; i += 256) {
+      const int m = i / HW_BK, k = i % HW_BK;
+      xs[m][k] = (m0 + m < rows && k0 + k < n_in)
+                     ? to_f32(x[(size_t)(m0 + m) * x_row + (size_t)h * x_head + k0 + k]) : 0.f;
+    }
+    for (int i = tid; i < HW_BN * HW_BK; i += 256) {
+      const int n = i / HW_BK, k = i % HW_BK;
+      ws[n][k] = (n0 + n < n_out && k0 + k < n_in) ? to_f32(wh[(size_t)(n0 + n) * n_in + k0 + k])
+                                                   : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 8
+    for (int k = 0; k < HW_BK; ++k) {
+      const float a0 = xs[2 * ty][k], a1 = xs[2 * ty + 1][k];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float b = ws[4 * tx + j][k];
+        acc[0][j] = fmaf(a0, b, acc[0][j]);
+        acc[1][j] = fmaf(a1, b, acc[1][j]);
+      }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int m = m0 + 2 * ty + i;
+    if (m >= rows) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + 4 * tx + j;
+      if (n < n_out) from_f32(y + (size_t)m * y_row + (size_t)h * y_head + n, acc[i][j]);
+    }
+  }
+}
+
+extern "C" int kappai_headwise_linear(const void* x, int x_row, int x_head, const void* w, int H,
+                                      int n_out, int n_in, void* y, int y_row, int y_head,
+                                      int rows, int is_bf16, hipStream_t stream) {
+  if (rows <= 0) return 0;
+  if (H < 1 || H > 65535 || n_out < 1 || n_in < 1) return (int)hipErrorInvalidValue;
+  dim3 grid((rows + HW_BM - 1) / HW_BM, (n_out + HW_BN - 1) / HW_BN, H);
+  if (grid.y > 65535) return (int)hipErrorInvalidValue;
+  if (is_bf16)
+    hipLaunchKernelGGL(headwise_linear_kernel<bf16_t>, grid, dim3(256), 0, stream,
+                       (const bf16_t*)x, x_row, x_head, (const bf16_t*)w, n_out, n_in, (bf16_t*)y,
+                       y_row, y_head, rows);
+  else
+    hipLaunchKernelGGL(headwise_linear_kernel<float>, grid, dim3(256), 0, stream, (const float*)x,
+                       x_row, x_head, (const float*)w, n_out, n_in, (float*)y, y_row, y_head, rows);
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}

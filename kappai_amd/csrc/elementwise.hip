@@ -59,6 +59,60 @@ extern "C" int kappai_embed_rows(const int* ids, const void* table, int table_is
 }
 
 // ---------------------------------------------------------------------------------------
+// A norm on what a sublayer returns: y = scale_a * a (+ scale_b * b), n = y / sqrt(mean(y^2) + eps)
+// * w, then resid += n (or resid = n), and the new resid again in the compute dtype for the next
+// sublayer to read.  a may come as `a_parts` float planes [parts][T][D] that are added in order
+// first (a product cut over its input dimension).  Everything in float32; a block a row, the row
+// kept in LDS between the sum of squares and the scaling.
+// ---------------------------------------------------------------------------------------
+template <typename TA, typename TO>
+__global__ __launch_bounds__(256) void output_norm_add_kernel(
+    const TA* __restrict__ a, int a_parts, size_t a_plane, float scale_a, const TA* __restrict__ b,
+    float scale_b, const float* __restrict__ w, float eps, float* __restrict__ resid, int add,
+    TO* __restrict__ rows, int D) {
+  extern __shared__ float ys[];
+  __shared__ float red[16];
+  const size_t at = (size_t)blockIdx.x * D;
+  float ss = 0.f;
+  for (int e = threadIdx.x; e < D; e += 256) {
+    float v = to_f32(a[at + e]);
+    for (int k = 1; k < a_parts; ++k) v += to_f32(a[k * a_plane + at + e]);
+    v *= scale_a;
+    if (b != nullptr) v = fmaf(scale_b, to_f32(b[at + e]), v);
+    ys[e] = v;
+    ss = fmaf(v, v, ss);
+  }
+  const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)D + eps);
+  for (int e = threadIdx.x; e < D; e += 256) {
+    float n = ys[e] * inv * w[e];
+    if (add) n += resid[at + e];
+    resid[at + e] = n;
+    if (rows != nullptr) from_f32(rows + at + e, n);
+  }
+}
+
+extern "C" int kappai_output_norm_add(const void* a, int a_is_bf16, int a_parts, float scale_a,
+                                      const void* b, float scale_b, const float* w, float eps,
+                                      float* resid, int add, void* rows, int rows_is_bf16, int T,
+                                      int D, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (D < 1 || D > 15 * 1024 || a_parts < 1 || (a_is_bf16 && a_parts != 1))
+    return (int)hipErrorInvalidValue;
+  const size_t lds = (size_t)D * sizeof(float), plane = (size_t)T * D;
+#define KAPPAI_OUT_NORM(TA, TO)                                                                  \
+  hipLaunchKernelGGL((output_norm_add_kernel<TA, TO>), dim3(T), dim3(256), lds, stream,          \
+                     (const TA*)a, a_parts, plane, scale_a, (const TA*)b, scale_b, w, eps, resid, \
+                     add, (TO*)rows, D)
+  if (a_is_bf16) {
+    if (rows_is_bf16) KAPPAI_OUT_NORM(bf16_t, bf16_t); else KAPPAI_OUT_NORM(bf16_t, float);
+  } else {
+    if (rows_is_bf16) KAPPAI_OUT_NORM(float, bf16_t); else KAPPAI_OUT_NORM(float, float);
+  }
+#undef KAPPAI_OUT_NORM
+  KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+// ---------------------------------------------------------------------------------------
 // tokens[dst_rows[i]] = chosen[src_idx[i]]: token ids that the last step's sampling kernels
 // left on the GPU go to their rows of this step's token table without a trip through the host.
 // ---------------------------------------------------------------------------------------

@@ -26,6 +26,7 @@ from ..cache.manager import CacheManager, RequestCache
 from .batch import StepEntry
 
 MAX_LIVE_REQUESTS = 8          # state slots of the replay pool (a trace has up to four live)
+TRACE_SLOTS = 4                # what the command line makes unless told otherwise
 REPLAY_PAGE_SIZE = 16          # divides the 64 that a request's token count is rounded up to
 
 
@@ -92,6 +93,8 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens that live requests hold at any time")
     ap.add_argument("--page-size", type=int, default=REPLAY_PAGE_SIZE)
+    ap.add_argument("--slots", type=int, default=TRACE_SLOTS,
+                    help="state slots: the most requests that are live at any time")
     ap.add_argument("--device", default="cuda:0")
     args = ap.parse_args(argv)
 
@@ -104,7 +107,7 @@ def main(argv=None) -> int:
         print("trace_run: no GPU is visible; kappai_amd runs on the GPU only", file=sys.stderr)
         return 1
     model = load_model(args.model, args.dtype, args.device)
-    cache = make_replay_cache(model, args.max_tokens, args.page_size)
+    cache = make_replay_cache(model, args.max_tokens, args.page_size, args.slots)
     cache.allocate_storage(model.dtype, args.device)
     runner = StepRunner(model, cache, args.device)
     rep = TraceReplayer(runner, args.out)

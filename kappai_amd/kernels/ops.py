@@ -809,6 +809,41 @@ def qk_norm_rope_store(qkv: torch.Tensor, n_heads: int, n_kv_heads: int, head_di
     return qkv if parts is None else q_out
 
 
+class ScoreModsC(ctypes.Structure):
+    """``kappai_score_mods`` of csrc/score_mods.h."""
+    _fields_ = [("softcap", _c_float), ("dist_bias", _vp), ("dist_cols", _c_int), ("sink", _vp)]
+
+
+@dataclass(frozen=True)
+class ScoreMods:
+    """What the attention kernels do to a score between the scaled dot product and the softmax:
+    ``softcap`` (0: nothing; else ``softcap * tanh(score / softcap)``); ``distance_bias`` float32
+    [H, n], added after the cap, column ``min(i - j, n - 1)`` for query position i and key
+    position j; ``sink`` float32 [H]: ``exp(sink[h])`` joins the softmax's denominator once, with
+    no key and no value behind it."""
+    softcap: float = 0.0
+    distance_bias: Optional[torch.Tensor] = None
+    sink: Optional[torch.Tensor] = None
+
+    def active(self) -> bool:
+        return self.softcap > 0.0 or self.distance_bias is not None or self.sink is not None
+
+    def c_struct(self, n_heads: int) -> "ScoreModsC":
+        cols = 0
+        if self.distance_bias is not None:
+            _gpu("distance_bias", self.distance_bias, F32)
+            _need(self.distance_bias.dim() == 2 and self.distance_bias.shape[0] == n_heads
+                  and self.distance_bias.shape[1] >= 1,
+                  lambda: f"distance_bias {tuple(self.distance_bias.shape)} for {n_heads} heads")
+            cols = self.distance_bias.shape[1]
+        if self.sink is not None:
+            _gpu("sink", self.sink, F32)
+            _need(self.sink.shape == (n_heads,), lambda: f"sink {tuple(self.sink.shape)}")
+        return ScoreModsC(float(self.softcap),
+                          0 if self.distance_bias is None else self.distance_bias.data_ptr(), cols,
+                          0 if self.sink is None else self.sink.data_ptr())
+
+
 @dataclass
 class QkPrologue:
     """What the decode attention kernels do themselves when they are given the projection as it
@@ -850,7 +885,8 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
                     single_rows: bool = False, max_position: Optional[int] = None,
                     kernel: str = "auto", prefill_variant: int = 0,
                     qk: Optional[QkPrologue] = None, lone_rows: Optional[torch.Tensor] = None,
-                    max_lone_position: int = -1) -> torch.Tensor:
+                    max_lone_position: int = -1,
+                    mods: Optional[ScoreMods] = None) -> torch.Tensor:
     """Causal attention of every row over the keys of its request that are in the cache
     (its own included; the last ``window`` of them when a window is set).  ``q`` is
     [T, >= H d] with a row stride (the q columns of the fused projection).  Returns [T, H d].
@@ -870,8 +906,14 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
 
     ``lone_rows`` (int32, with ``max_lone_position``; tiled kernel only): rows that ``q_tiles``
     leaves out, the single decoded tokens of a step that also holds prompt portions.  They go
-    through the decode kernel that splits keys over blocks."""
+    through the decode kernel that splits keys over blocks.
+
+    ``mods`` (``ScoreMods``): a cap on the scores, a bias by distance, a sink."""
     H, G, d = n_heads, n_kv_heads, head_dim
+    if mods is not None and not mods.active():
+        mods = None
+    mods_c = mods.c_struct(H) if mods is not None else None
+    mods_ref = ctypes.byref(mods_c) if mods_c is not None else None
     _gpu("q", q, (F32, BF16), contiguous=False)
     T = q.shape[0]
     _need(q.dim() == 2 and q.shape[1] >= H * d and (q.stride(1) == 1),
@@ -899,12 +941,15 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
             kernel = "prefill"
         else:
             kernel = "rows"
+    if mods is not None:
+        kernel = "rows"            # (the only kernel that knows them yet)
     if kernel == "rows":
-        check(library("attention").kappai_paged_attention_rows(
+        check(library("attention").kappai_paged_attention_rows_scored(
             _ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
             _ptr(row_pos), _ptr(row_seg), _ptr(block_tables), _c_int(block_tables.shape[1]),
             _c_int(T), _c_int(H), _c_int(G), _c_int(d), _c_int(page_size), _c_int(window or 0),
-            _c_float(scale), _c_int(_is_bf16(q.dtype)), _stream()), "paged_attention_rows")
+            _c_float(scale), _c_int(_is_bf16(q.dtype)), mods_ref, _stream()),
+            "paged_attention_rows")
         return out
     _need(mfma_ok, "the matrix-core attention kernels need bfloat16, a page size and a head size "
           f"that are multiples of 16 (head size at most 256) and 16-byte aligned rows; got "
@@ -1561,4 +1606,276 @@ def moe_combine(y: torch.Tensor, weights: torch.Tensor, plan: MoePlan) -> torch.
     check(library("moe").kappai_moe_combine(
         _ptr(y), _ptr(plan.slot_of_pair), _ptr(weights), _c_int(T), _c_int(top), _c_int(D),
         _ptr(out), _stream()), "moe_combine")
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+# a norm on a sublayer's output, added into the residual stream
+# ---------------------------------------------------------------------------------------
+def output_norm_add(resid: torch.Tensor, a: torch.Tensor, weight: torch.Tensor, eps: float,
+                    rows_dtype=None, scale_a: float = 1.0, b: Optional[torch.Tensor] = None,
+                    scale_b: float = 1.0, add: bool = True) -> Optional[torch.Tensor]:
+    """``y = scale_a a (+ scale_b b)``; ``resid (+)= y / sqrt(mean(y^2) + eps) * weight`` in
+    float32, in place (``add`` False: the residual becomes the normalised rows).  ``a``: [T, D]
+    in float32 or bfloat16, or float32 partial sums [S, T, D], added in order first; ``b`` like
+    ``a`` but always [T, D].  With ``rows_dtype`` the new residual is also returned rounded to that
+    dtype, for the next sublayer to read."""
+    _gpu("resid", resid, F32)
+    _gpu("a", a, (F32, BF16))
+    _gpu("weight", weight, F32)
+    T, D = resid.shape
+    parts = 1
+    if a.dim() == 3:
+        _need(a.dtype == F32, "output_norm_add: partial sums are float32")
+        parts = a.shape[0]
+    _need(tuple(a.shape[-2:]) == (T, D) and weight.shape == (D,),
+          lambda: f"output_norm_add: {tuple(a.shape)} into {tuple(resid.shape)}")
+    if b is not None:
+        _gpu("b", b, a.dtype)
+        _need(tuple(b.shape) == (T, D), lambda: f"output_norm_add: b {tuple(b.shape)}")
+    rows = None
+    if rows_dtype is not None:
+        rows = torch.empty((T, D), dtype=rows_dtype, device=resid.device)
+    check(library("elementwise").kappai_output_norm_add(
+        _ptr(a), _c_int(_is_bf16(a.dtype)), _c_int(parts), _c_float(scale_a), _ptr(b),
+        _c_float(scale_b), _ptr(weight), _c_float(eps), _ptr(resid), _c_int(1 if add else 0),
+        _ptr(rows), _c_int(_is_bf16(rows_dtype) if rows is not None else 0), _c_int(T), _c_int(D),
+        _stream()), "output_norm_add")
+    return rows
+
+
+# ---------------------------------------------------------------------------------------
+# attention layers whose queries, keys and values are not the plain grouped-query form
+# ---------------------------------------------------------------------------------------
+def projection_norm_store(proj: torch.Tensor, n_heads: int, n_kv_heads: int, dim: int, vdim: int,
+                          head_size: int, q_norm_w: Optional[torch.Tensor],
+                          k_norm_w: Optional[torch.Tensor], eps: float, temp_coef: float,
+                          temp_every: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                          row_pos: torch.Tensor, row_seg: torch.Tensor,
+                          block_tables: torch.Tensor, page_size: int,
+                          store_kv: bool = True) -> torch.Tensor:
+    """From ``proj`` [T, H dim + G dim + G vdim]: q and k each divided by the root mean square of
+    their WHOLE projection (all heads together) and multiplied by weights [H dim] / [G dim]
+    (None: no norm); q also by ``1 + temp_coef * ln(floor((position + 1) / temp_every) + 1)``.
+    Returns queries [T, H head_size] (zeros behind ``dim``); keys and values go to pools made for
+    G kv heads of ``head_size`` (``PagedKV``)."""
+    H, G, d, dv, D = n_heads, n_kv_heads, dim, vdim, head_size
+    _gpu("proj", proj, (F32, BF16), contiguous=False)
+    T = proj.shape[0]
+    need = H * d + G * d + G * dv
+    _need(proj.dim() == 2 and proj.shape[1] >= need and proj.stride(1) == 1,
+          lambda: f"projection_norm_store: proj {tuple(proj.shape)} holds fewer than {need} columns")
+    _need(H % G == 0 and d <= D and dv <= D and temp_every >= 1,
+          lambda: f"projection_norm_store: {H} heads over {G}, sizes {d} and {dv} in heads of {D}")
+    for name, w, n in (("q_norm_w", q_norm_w, H * d), ("k_norm_w", k_norm_w, G * d)):
+        if w is not None:
+            _gpu(name, w, F32)
+            _need(w.shape == (n,), lambda: f"{name}: {tuple(w.shape)}, expected ({n},)")
+    _gpu("row_pos", row_pos, I32)
+    _gpu("row_seg", row_seg, I32)
+    max_blocks = 0
+    if store_kv:
+        _gpu("k_pool", k_pool, proj.dtype)
+        _gpu("v_pool", v_pool, proj.dtype)
+        _gpu("block_tables", block_tables, I32)
+        _check_pools(k_pool, v_pool, G, page_size, D)
+        max_blocks = block_tables.shape[1]
+    q = torch.empty((T, H * D), dtype=proj.dtype, device=proj.device)
+    check(library("attn_prep").kappai_projection_norm_store(
+        _ptr(proj), _c_int(proj.stride(0)), _ptr(q_norm_w), _ptr(k_norm_w), _c_float(eps),
+        _c_float(temp_coef), _c_int(temp_every), _ptr(k_pool if store_kv else None),
+        _ptr(v_pool if store_kv else None), _ptr(row_pos), _ptr(row_seg),
+        _ptr(block_tables if store_kv else None), _c_int(max_blocks), _c_int(T), _c_int(H),
+        _c_int(G), _c_int(d), _c_int(dv), _c_int(D), _c_int(page_size), _ptr(q),
+        _c_int(_is_bf16(proj.dtype)), _stream()), "projection_norm_store")
+    return q
+
+
+def latent_store(q: torch.Tensor, kv: torch.Tensor, n_heads: int, dim: int, rot_dim: int,
+                 rank: int, head_size: int, c_norm_w: torch.Tensor, eps: float,
+                 cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], rot_dims: int,
+                 rot_mode: int, k_pool: torch.Tensor, v_pool: torch.Tensor,
+                 row_pos: torch.Tensor, row_seg: torch.Tensor, block_tables: torch.Tensor,
+                 page_size: int) -> torch.Tensor:
+    """``kv`` [T, rank + rot_dim]: the first ``rank`` entries, RMS-normed with ``c_norm_w``, are
+    the token's latent; the rest is a key part that is rotated by the position.  They are stored
+    as the one kv head's key ``[latent | rotated | 0]`` of ``head_size``, the latent again as its
+    value.  ``q`` [T, H (dim + rot_dim)], head by head ``[dim | rot_dim]``: returns
+    [T, H head_size] whose places ``rank .. rank + rot_dim`` of every head hold the rotated part
+    (zeros behind); the first ``rank`` places are left for ``headwise_linear``."""
+    H, d, rot, r, D = n_heads, dim, rot_dim, rank, head_size
+    _gpu("q", q, (F32, BF16), contiguous=False)
+    _gpu("kv", kv, q.dtype, contiguous=False)
+    T = q.shape[0]
+    _need(q.dim() == 2 and q.shape[1] >= H * (d + rot) and q.stride(1) == 1 and kv.dim() == 2
+          and kv.shape[0] == T and kv.shape[1] >= r + rot and kv.stride(1) == 1,
+          lambda: f"latent_store: q {tuple(q.shape)}, kv {tuple(kv.shape)}")
+    _need(D >= r + rot and rot_dims <= rot and rot_dims % 2 == 0,
+          lambda: f"latent_store: a latent of {r} and {rot} rotated places in heads of {D}")
+    _gpu("c_norm_w", c_norm_w, F32)
+    _need(c_norm_w.shape == (r,), "latent_store: one norm weight for each entry of the latent")
+    if rot_mode != ROT_NONE and rot_dims:
+        _gpu("cos", cos, F32)
+        _gpu("sin", sin, F32)
+        _need(cos.shape == sin.shape and cos.dim() == 2 and cos.shape[1] == rot_dims // 2,
+              lambda: f"latent_store: rotation tables {tuple(cos.shape)} for {rot_dims} places")
+    _gpu("k_pool", k_pool, q.dtype)
+    _gpu("v_pool", v_pool, q.dtype)
+    _check_pools(k_pool, v_pool, 1, page_size, D)
+    for name, t in (("row_pos", row_pos), ("row_seg", row_seg), ("block_tables", block_tables)):
+        _gpu(name, t, I32)
+    out = torch.empty((T, H * D), dtype=q.dtype, device=q.device)
+    check(library("attn_prep").kappai_latent_store(
+        _ptr(q), _c_int(q.stride(0)), _ptr(kv), _c_int(kv.stride(0)), _ptr(c_norm_w),
+        _c_float(eps), _ptr(cos), _ptr(sin), _c_int(rot_dims), _c_int(rot_mode), _ptr(k_pool),
+        _ptr(v_pool), _ptr(row_pos), _ptr(row_seg), _ptr(block_tables),
+        _c_int(block_tables.shape[1]), _c_int(T), _c_int(H), _c_int(d), _c_int(rot), _c_int(r),
+        _c_int(D), _c_int(page_size), _ptr(out), _c_int(_is_bf16(q.dtype)), _stream()),
+        "latent_store")
+    return out
+
+
+def headwise_linear(x: torch.Tensor, x_head_stride: int, weight: torch.Tensor,
+                    out: Optional[torch.Tensor] = None, out_head_stride: Optional[int] = None
+                    ) -> torch.Tensor:
+    """``y[t, h, :] = weight[h] @ x[t, h, :]`` with ``weight`` [H, n_out, n_in] in the dtype of
+    ``x``.  Head h of row t starts at ``x[t, h * x_head_stride]`` and is written at
+    ``out[t, h * out_head_stride]`` (``out`` None: a new [T, H n_out])."""
+    _gpu("x", x, (F32, BF16), contiguous=False)
+    _gpu("weight", weight, x.dtype)
+    _need(weight.dim() == 3, "headwise_linear: weight must be [heads, out, in]")
+    H, n_out, n_in = weight.shape
+    T = x.shape[0]
+    _need(x.dim() == 2 and x.stride(1) == 1 and (H - 1) * x_head_stride + n_in <= x.shape[1],
+          lambda: f"headwise_linear: x {tuple(x.shape)} for {H} heads of {n_in} every "
+                  f"{x_head_stride}")
+    if out is None:
+        out = torch.empty((T, H * n_out), dtype=x.dtype, device=x.device)
+        out_head_stride = n_out
+    _gpu("out", out, x.dtype, contiguous=False)
+    _need(out.dim() == 2 and out.shape[0] == T and out.stride(1) == 1
+          and (H - 1) * out_head_stride + n_out <= out.shape[1],
+          lambda: f"headwise_linear: out {tuple(out.shape)}")
+    check(library("attn_prep").kappai_headwise_linear(
+        _ptr(x), _c_int(x.stride(0)), _c_int(x_head_stride), _ptr(weight), _c_int(H),
+        _c_int(n_out), _c_int(n_in), _ptr(out), _c_int(out.stride(0)), _c_int(out_head_stride),
+        _c_int(T), _c_int(_is_bf16(x.dtype)), _stream()), "headwise_linear")
+    return out
+
+
+# ---------------------------------------------------------------------------------------
+# recurrences with a matrix of state per head
+# ---------------------------------------------------------------------------------------
+CONV_SILU_MAX_TAPS = 17
+
+
+def conv_silu(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, row_pos: torch.Tensor,
+              row_seg: torch.Tensor, seg_start: torch.Tensor, seg_pos0: torch.Tensor,
+              seg_slot: torch.Tensor) -> torch.Tensor:
+    """``silu(conv(x))`` per channel: ``conv(x)[t] = sum_j taps[:, j] x[t - n + 1 + j]``, zeros
+    before position 0.  ``x`` [T, >= C] (a view with a row stride), ``taps`` [C, n] float32,
+    ``state`` [slots, n - 1, C] float32: the request's last inputs, read for rows before the
+    step's portion and brought up to date.  Returns [T, C] in the dtype of ``x``."""
+    _gpu("x", x, (F32, BF16), contiguous=False)
+    _gpu("taps", taps, F32)
+    _gpu("state", state, F32)
+    C, n = taps.shape
+    T = x.shape[0]
+    _need(x.dim() == 2 and x.shape[1] >= C and x.stride(1) == 1,
+          lambda: f"conv_silu: x {tuple(x.shape)} for {C} channels")
+    _need(1 <= n <= CONV_SILU_MAX_TAPS and tuple(state.shape[1:]) == (n - 1, C),
+          lambda: f"conv_silu: {n} taps, state {tuple(state.shape)}")
+    for name, t in (("row_pos", row_pos), ("row_seg", row_seg), ("seg_start", seg_start),
+                    ("seg_pos0", seg_pos0), ("seg_slot", seg_slot)):
+        _gpu(name, t, I32)
+    S = seg_slot.shape[0]
+    out = torch.empty((T, C), dtype=x.dtype, device=x.device)
+    check(library("linear_attention").kappai_conv_silu(
+        _ptr(x), _c_int(x.stride(0)), _ptr(taps), _c_int(n), _ptr(state), _ptr(row_pos),
+        _ptr(row_seg), _ptr(seg_start), _ptr(seg_pos0), _ptr(seg_slot), _c_int(T), _c_int(S),
+        _c_int(C), _ptr(out), _c_int(_is_bf16(x.dtype)), _stream()), "conv_silu")
+    return out
+
+
+def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor,
+                            n_heads: int, n_qk_heads: int, dim: int, vdim: int,
+                            rate: torch.Tensor, z_bias: Optional[torch.Tensor], z_sign: float,
+                            q_scale: float, state: torch.Tensor, seg_start: torch.Tensor,
+                            seg_pos0: torch.Tensor, seg_slot: torch.Tensor,
+                            beta: Optional[torch.Tensor] = None, unit_qk: bool = False,
+                            unit_eps: float = 1e-6) -> torch.Tensor:
+    """A state ``S`` [dim, vdim] per head, float32, in ``state`` [slots, H, dim, vdim] (a segment
+    that starts at position 0 starts from zero).  Per token, with the decay per key channel
+    ``a = exp(-rate[h] * softplus(z_sign * (z + z_bias)))``:
+    without ``beta``   ``S <- diag(a) S + k v^T``, ``o = S^T q``;
+    with ``beta``      ``S <- diag(a) S``, ``u = sigmoid(beta) (v - S^T k)``, ``S <- S + k u^T``,
+                       ``o = S^T q`` (the delta rule; the read-out sees the token's own write).
+    ``q``, ``k`` [T, Hk dim] (head h reads q/k head ``h // (H / Hk)``; ``unit_qk``: each head's
+    vector divided by ``sqrt(sum x^2 + unit_eps)`` first), q times ``q_scale``; ``v`` [T, H vdim];
+    ``z`` [T, H dim]; ``beta`` [T, H]; all views with a row stride.  Everything between the
+    projections and the result is float32.  Returns ``o`` [T, H vdim] float32."""
+    H, Hk, d, dv = n_heads, n_qk_heads, dim, vdim
+    T = q.shape[0]
+    for name, t, cols in (("q", q, Hk * d), ("k", k, Hk * d), ("v", v, H * dv), ("z", z, H * d)):
+        _gpu(name, t, q.dtype, contiguous=False)
+        _need(t.dim() == 2 and t.shape[0] == T and t.shape[1] >= cols and t.stride(1) == 1,
+              lambda: f"matrix_state_recurrence: {name} {tuple(t.shape)}, expected [T, {cols}]")
+    _need(q.dtype in (F32, BF16) and H % Hk == 0, "matrix_state_recurrence: dtypes / heads")
+    if beta is not None:
+        _gpu("beta", beta, q.dtype, contiguous=False)
+        _need(beta.dim() == 2 and beta.shape[0] == T and beta.shape[1] >= H
+              and (beta.stride(1) == 1 or H == 1), "matrix_state_recurrence: beta must be [T, H]")
+    _gpu("rate", rate, F32)
+    _need(rate.shape == (H,), "matrix_state_recurrence: one rate a head")
+    if z_bias is not None:
+        _gpu("z_bias", z_bias, F32)
+        _need(z_bias.shape == (H * d,), "matrix_state_recurrence: z_bias must be [H dim]")
+    _gpu("state", state, F32)
+    _need(tuple(state.shape[1:]) == (H, d, dv),
+          lambda: f"matrix_state_recurrence: state {tuple(state.shape)} for {H} x {d} x {dv}")
+    for name, t in (("seg_start", seg_start), ("seg_pos0", seg_pos0), ("seg_slot", seg_slot)):
+        _gpu(name, t, I32)
+    S = seg_slot.shape[0]
+    dev = q.device
+    qf = torch.empty((T, Hk * d), dtype=F32, device=dev)
+    kf = torch.empty((T, Hk * d), dtype=F32, device=dev)
+    af = torch.empty((T, H * d), dtype=F32, device=dev)
+    bf = torch.empty((T, H), dtype=F32, device=dev) if beta is not None else None
+    lib = library("linear_attention")
+    check(lib.kappai_recurrence_prep(
+        _ptr(q), _c_int(q.stride(0)), _ptr(k), _c_int(k.stride(0)), _ptr(z), _c_int(z.stride(0)),
+        _ptr(z_bias), _ptr(rate), _c_float(z_sign), _ptr(beta),
+        _c_int(beta.stride(0) if beta is not None else 0), _c_int(T), _c_int(H), _c_int(Hk),
+        _c_int(d), _c_int(1 if unit_qk else 0), _c_float(unit_eps), _c_float(q_scale), _ptr(qf),
+        _ptr(kf), _ptr(af), _ptr(bf), _c_int(_is_bf16(q.dtype)), _stream()), "recurrence_prep")
+    out = torch.empty((T, H * dv), dtype=F32, device=dev)
+    check(lib.kappai_matrix_state_scan(
+        _ptr(qf), _ptr(kf), _ptr(af), _ptr(bf), _ptr(v), _c_int(v.stride(0)),
+        _c_int(_is_bf16(v.dtype)), _ptr(state), _ptr(seg_start), _ptr(seg_pos0), _ptr(seg_slot),
+        _c_int(T), _c_int(S), _c_int(H), _c_int(Hk), _c_int(d), _c_int(dv),
+        _c_int(1 if beta is not None else 0), _ptr(out), _stream()), "matrix_state_scan")
+    return out
+
+
+GATE_SILU, GATE_SIGMOID = 0, 1
+
+
+def head_norm_gate(o: torch.Tensor, weight: torch.Tensor, eps: float, gate: torch.Tensor,
+                   gate_kind: int, n_heads: int, vdim: int, out_dtype) -> torch.Tensor:
+    """Per head ``o / sqrt(mean(o^2) + eps) * weight`` (``weight`` [vdim], shared by the heads)
+    times ``silu(gate)`` or ``sigmoid(gate)``: ``o`` [T, H vdim] float32, ``gate`` [T, >= H vdim]
+    in ``out_dtype`` (a view with a row stride).  Returns [T, H vdim] in ``out_dtype``."""
+    H, dv = n_heads, vdim
+    _gpu("o", o, F32)
+    _gpu("weight", weight, F32)
+    _gpu("gate", gate, out_dtype, contiguous=False)
+    T = o.shape[0]
+    _need(tuple(o.shape) == (T, H * dv) and weight.shape == (dv,) and gate.dim() == 2
+          and gate.shape[0] == T and gate.shape[1] >= H * dv and gate.stride(1) == 1,
+          lambda: f"head_norm_gate: o {tuple(o.shape)}, gate {tuple(gate.shape)}")
+    out = torch.empty((T, H * dv), dtype=out_dtype, device=o.device)
+    check(library("linear_attention").kappai_head_norm_gate(
+        _ptr(o), _ptr(weight), _c_float(eps), _ptr(gate), _c_int(gate.stride(0)),
+        _c_int(gate_kind), _c_int(T), _c_int(H), _c_int(dv), _ptr(out),
+        _c_int(_is_bf16(out_dtype)), _stream()), "head_norm_gate")
     return out

@@ -30,11 +30,15 @@ class Model:
     def __init__(self, config: ModelConfig, dtype: torch.dtype, embedding: TokenEmbedding,
                  layers: Sequence[Block], final_norm: Norm, head: OutputHead,
                  schedule: Optional[Sequence[LayerCall]] = None,
-                 embedding_position: Optional[PositionEncoding] = None):
+                 embedding_position: Optional[PositionEncoding] = None,
+                 embedding_norm: Optional[Norm] = None):
+        """``embedding_norm``: a norm that the embedded rows pass before the first layer (one with
+        ``norm_output``); the stream then starts as the normalised rows."""
         self.config, self.dtype = config, dtype
         self.embedding, self.layers = embedding, list(layers)
         self.final_norm, self.head = final_norm, head
         self.embedding_position = embedding_position
+        self.embedding_norm = embedding_norm
         # names a checkpoint may hold although this model reads none of them (a builder fills it)
         self.unused_tensor_names: List[str] = []
         self.schedule: List[LayerCall] = list(schedule) if schedule is not None else [
@@ -75,6 +79,8 @@ class Model:
         parts = [self.embedding, *self.layers, self.final_norm, self.head]
         if self.embedding_position is not None:
             parts.append(self.embedding_position)
+        if self.embedding_norm is not None:
+            parts.append(self.embedding_norm)
         return parts
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -135,6 +141,8 @@ class Model:
         changes ``forward`` gets no walk from C unless it describes one."""
         from ..parts.cdesc import defined_together
         calls = []
+        if self.embedding_norm is not None:
+            return None            # the walk from C knows no norm between embedding and layers
         for ci, call in enumerate(self.schedule):
             block = self.layers[call.layer]
             if not defined_together(block, "forward", "c_call"):
@@ -157,6 +165,10 @@ class Model:
         if self.embedding_position is not None:
             self.embedding_position.on_embedding(x, batch)
         h = Hidden(x, None)
+        if self.embedding_norm is not None:
+            narrow = self.dtype != torch.float32
+            h.rows = self.embedding_norm.norm_output(x, x, add=False,
+                                                     rows_dtype=self.dtype if narrow else None)
         for ci, call in enumerate(self.schedule):
             block = self.layers[call.layer]
             view = None

@@ -1,18 +1,22 @@
 from .attention import GroupedQueryAttention
 from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Block, FeedForward,
                    Hidden, Mixer, Norm, Part, PositionEncoding, make_part, register_part)
-from .block import ConvInputBlock, PreNormBlock
+from .block import ConvInputBlock, OutputNormBlock, PreNormBlock
 from .diff_attention import DifferentialAttention
 from .embedding import OutputHead, TokenEmbedding
 from .feed_forward import SwiGLU
 from .group_norm import GroupRMSNorm
 from .input_conv import ShortInputConv
+from .latent_attention import LatentAttention
 from .linear import Linear
+from .linear_attention import GatedDeltaRule, GatedLinearAttention
 from .mingru import MinGRU
 from .moe import MixtureOfExperts
 from .norm import RMSNorm
+from .parallel import ParallelMixer
 from .positions import LearnedPositions
 from .rotary import RotaryEncoding, Rotation
+from .scored_attention import ScoredAttention
 from .shortconv import GatedShortConv
 
 __all__ = ["GroupedQueryAttention", "BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS",
@@ -20,4 +24,6 @@ __all__ = ["GroupedQueryAttention", "BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS"
            "PositionEncoding", "make_part", "register_part", "PreNormBlock", "OutputHead",
            "TokenEmbedding", "SwiGLU", "Linear", "RMSNorm", "RotaryEncoding", "Rotation",
            "GatedShortConv", "ConvInputBlock", "DifferentialAttention", "GroupRMSNorm",
-           "ShortInputConv", "MinGRU", "MixtureOfExperts", "LearnedPositions"]
+           "ShortInputConv", "MinGRU", "MixtureOfExperts", "LearnedPositions", "OutputNormBlock",
+           "LatentAttention", "GatedDeltaRule", "GatedLinearAttention", "ParallelMixer",
+           "ScoredAttention"]

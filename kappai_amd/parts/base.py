@@ -159,9 +159,22 @@ class Hidden:
     """The residual stream between blocks: ``resid`` (float32, [T, width]) and the last
     part's output ``delta`` that has not been added yet ([T, width], or float32 partial sums
     [S, T, width]).  The next norm adds it while it normalises, so the sum is made in float32
-    and costs no pass of its own."""
+    and costs no pass of its own.  ``rows``: the stream rounded to the compute dtype, when the
+    kernel that last changed it wrote that too (arrangements whose sublayers read the stream
+    itself)."""
     resid: torch.Tensor
     delta: Optional[object] = None      # a tensor, or ops.Added / ops.ScaledRows: nothing to add
+    rows: Optional[torch.Tensor] = None
+
+
+@dataclass
+class WeightedTerms:
+    """What a mixer made of two returns: ``scale_a * a + scale_b * b``, not summed yet (the norm
+    or the sum that follows does it in float32).  ``a`` and ``b``: [T, width] in one dtype."""
+    a: torch.Tensor
+    scale_a: float
+    b: torch.Tensor
+    scale_b: float
 
 
 class Block(Part):

@@ -201,3 +201,67 @@ class ConvInputBlock(Block):
 
 
 register_part("block", "conv_input", ConvInputBlock)
+
+
+class OutputNormBlock(Block):
+    """``x += norm1(mixer(x)); x += norm2(feed_forward(x))``: the sublayers read the stream itself
+    and the norm sits on what they return.  ``feed_forward`` (with its norm) may be None.  The
+    stream is float32; the kernel that adds a normalised result also writes the stream rounded to
+    the compute dtype, which is what the next sublayer reads (``Hidden.rows``).  The norms are
+    RMS norms that know ``norm_output`` (``parts.norm.RMSNorm``)."""
+
+    def __init__(self, mixer: Mixer, mixer_norm: Norm, feed_forward=None, ffn_norm=None):
+        if (feed_forward is None) != (ffn_norm is None):
+            raise ValueError("a feed-forward and its norm come together")
+        for n in (mixer_norm, ffn_norm):
+            if n is not None and not hasattr(n, "norm_output"):
+                raise ValueError(f"{type(n).__name__} cannot norm a sublayer's output into the "
+                                 "stream (no norm_output)")
+        self.mixer, self.mixer_norm = mixer, mixer_norm
+        self.feed_forward, self.ffn_norm = feed_forward, ffn_norm
+
+    def _parts(self):
+        return tuple(p for p in (self.mixer, self.mixer_norm, self.feed_forward, self.ffn_norm)
+                     if p is not None)
+
+    @property
+    def capturable(self) -> bool:
+        return all(p.capturable for p in self._parts())
+
+    @property
+    def step_tables(self):
+        out = []
+        for p in self._parts():
+            asked = p.step_tables
+            if asked is not None:
+                out += list(asked) if isinstance(asked, (list, tuple)) else [asked]
+        return out
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s for p in self._parts() for s in p.tensor_specs()]
+
+    def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for p in self._parts():
+            p.bind(tensors)
+
+    def forward(self, h: Hidden, batch, cache, shared_cache: bool = False) -> Hidden:
+        resid = h.resid
+        if h.delta is not None:
+            raise ValueError("the block before left an update that was not added to the stream")
+        narrow = self.mixer_norm.dtype != torch.float32
+        rows_dtype = self.mixer_norm.dtype if narrow else None
+        x = h.rows if narrow else resid
+        if x is None:
+            x = ops.cast(resid, self.mixer_norm.dtype)
+        mixed = self.mixer.forward(x, batch, cache, shared_cache=shared_cache)
+        rows = self.mixer_norm.norm_output(resid, mixed, rows_dtype=rows_dtype)
+        if self.feed_forward is not None:
+            out = self.feed_forward.forward(rows if narrow else resid, batch)
+            rows = self.ffn_norm.norm_output(resid, out, rows_dtype=rows_dtype)
+        return Hidden(resid, None, rows)
+
+    def weight_bytes(self) -> int:
+        return sum(p.weight_bytes() for p in self._parts())
+
+
+register_part("block", "output_norm", OutputNormBlock)

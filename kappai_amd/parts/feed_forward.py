@@ -30,9 +30,12 @@ class SwiGLU(FeedForward):
     ACTIVATIONS = {"silu": ops.GLU_SILU, "gelu_tanh": ops.GLU_GELU_TANH}
 
     def __init__(self, prefix: str, width: int, hidden: int, dtype: torch.dtype, names=None,
-                 activation: str = "silu", weight_suffix: str = ".weight"):
+                 activation: str = "silu", weight_suffix: str = ".weight", bias: bool = False,
+                 bias_suffix: str = ".bias"):
         """``activation``: what the gate passes through, "silu" or "gelu_tanh" (the tanh form of
-        GELU): ``W_down (act(W_gate x) * W_up x)``."""
+        GELU): ``W_down (act(W_gate x + b_gate) * (W_up x + b_up)) + b_down``; ``bias``: whether the
+        three maps have biases (the gate then runs as a kernel of its own behind the first
+        product, which adds the biases)."""
         n = {"gate": "w1", "up": "w3", "down": "w2"}
         n.update(names or {})
         if activation not in self.ACTIVATIONS:
@@ -41,10 +44,12 @@ class SwiGLU(FeedForward):
         self.width, self.hidden, self.dtype = width, hidden, dtype
         self.activation = activation
         self.fused = False
+        self.has_bias = bool(bias)
         self.gate_up = Linear([prefix + n["gate"], prefix + n["up"]], width, [hidden, hidden],
-                              stage="matmul_ffn_gate_up", weight_suffix=weight_suffix)
+                              stage="matmul_ffn_gate_up", weight_suffix=weight_suffix, bias=bias,
+                              bias_suffix=bias_suffix)
         self.down = Linear([prefix + n["down"]], hidden, [width], stage="matmul_ffn_down",
-                           weight_suffix=weight_suffix)
+                           weight_suffix=weight_suffix, bias=bias, bias_suffix=bias_suffix)
 
     def tensor_specs(self) -> List[TensorSpec]:
         return self.gate_up.tensor_specs() + self.down.tensor_specs()
@@ -53,7 +58,7 @@ class SwiGLU(FeedForward):
         def interleaved(w):
             # the fused product wants gate and up rows in turns of 16
             self.fused = (w.dtype == torch.bfloat16 and self.hidden % ops.SWIGLU_GROUP == 0
-                          and self.width % 8 == 0)
+                          and self.width % 8 == 0 and not self.has_bias)
             return ops.interleave_gate_up(w[:self.hidden], w[self.hidden:]) if self.fused else None
 
         self.gate_up.bind(tensors, arrange=interleaved)
@@ -69,13 +74,13 @@ class SwiGLU(FeedForward):
         with profile.scope("ffn_act"):
             act = (ops.swiglu(gate_up) if self.activation == "silu"
                    else ops.glu(gate_up, self.ACTIVATIONS[self.activation]))
-        return self.down.forward(act, partial_sums=True, add_into=into)
+        return self.down.forward(act, partial_sums=not self.has_bias, add_into=into)
 
     def c_part(self, plan, view=None, shared_cache: bool = False):
         """The runner "feed_forward.swiglu" (csrc/engine_parts.hip) makes the same choices as
         ``forward``."""
-        if self.activation != "silu":
-            return None            # the runner on the C side knows the SiLU gate only
+        if self.activation != "silu" or self.has_bias:
+            return None            # the runner on the C side knows the SiLU gate without biases only
         first = plan.linear(self.gate_up)
         desc = SwiGLUDesc(first, plan.linear(self.down), self.hidden, 1 if self.fused else 0)
         return plan.part("feed_forward.swiglu", desc, takes_deferred_rows=True,

@@ -8,8 +8,8 @@ from typing import Dict, List, Optional
 import torch
 
 from ..kernels import ops, profile, tuning
-from ..weights.spec import INIT_ONES, VECTOR, TensorSpec
-from .base import Norm, register_part
+from ..weights.spec import INIT_ONES, INIT_SMALL, VECTOR, TensorSpec
+from .base import Norm, WeightedTerms, register_part
 from .cdesc import FoldDesc
 
 
@@ -18,15 +18,38 @@ class RMSNorm(Norm):
     can_defer = True      # add_norm(..., defer=True) may hand out ops.ScaledRows or
                           # ops.FragmentRows in place of a tensor
 
-    def __init__(self, name: str, width: int, eps: float, dtype: torch.dtype):
+    def __init__(self, name: str, width: int, eps: float, dtype: torch.dtype,
+                 suffix: str = ".weight", weight_offset: float = 0.0, weight_scale: float = 1.0):
+        """``suffix``: how the weight's tensor name ends in the checkpoint.  ``weight_offset``: the
+        file stores the weight around zero and the norm multiplies by ``offset + w`` (1.0 for a
+        "one plus" weight).  ``weight_scale``: a constant factor on the normalised rows that the
+        owner wants folded in (a scale on the logits, for the norm before the head)."""
         self.name, self.width, self.eps, self.dtype = name, width, float(eps), dtype
+        self.tensor_name = name + suffix
+        self.weight_offset, self.weight_scale = float(weight_offset), float(weight_scale)
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [TensorSpec(self.name + ".weight", (self.width,), VECTOR, INIT_ONES)]
+        init = INIT_SMALL if self.weight_offset else INIT_ONES
+        return [TensorSpec(self.tensor_name, (self.width,), VECTOR, init)]
 
     def bind(self, tensors: Dict[str, torch.Tensor]) -> None:
-        self.weight = tensors[self.name + ".weight"].to(torch.float32).contiguous()
+        w = tensors[self.tensor_name].to(torch.float32)
+        if self.weight_offset or self.weight_scale != 1.0:
+            w = (w + self.weight_offset) * self.weight_scale
+        self.weight = w.contiguous()
+
+    def norm_output(self, resid, y, rows_dtype=None, add: bool = True):
+        """The norm on what a sublayer returned, added into the stream: ``resid += norm(y)`` in
+        float32, in place (``add`` False: ``resid = norm(y)``).  ``y``: [T, width], float32
+        partial sums [S, T, width], or ``WeightedTerms`` (two results and their weights, summed
+        here).  Returns the new stream rounded to ``rows_dtype`` (None: nothing)."""
+        a, sa, b, sb = y, 1.0, None, 1.0
+        if isinstance(y, WeightedTerms):
+            a, sa, b, sb = y.a, y.scale_a, y.b, y.scale_b
+        with profile.scope("rmsnorm"):
+            return ops.output_norm_add(resid, a, self.weight, self.eps, rows_dtype=rows_dtype,
+                                       scale_a=sa, b=b, scale_b=sb, add=add)
 
     def fold(self):
         """(weight, eps) for a product that folds this norm in (``ops.AddInto``): the norm is

@@ -76,6 +76,24 @@ def _weight_files(model_dir: Path) -> List[Path]:
     raise WeightsError(model_dir, [], [], [], [f"no model.safetensors in {model_dir}"])
 
 
+def tensor_shapes(model_dir) -> Dict[str, tuple]:
+    """``{name: shape}`` of every tensor of the folder's file(s), read from the headers alone: for
+    an architecture whose config.json leaves a size to the tensors' shapes."""
+    model_dir = Path(model_dir)
+    shapes: Dict[str, tuple] = {}
+    try:
+        for p in _weight_files(model_dir):
+            f = SafetensorsFile(p)
+            try:
+                for n in f.names():
+                    shapes[n] = tuple(f.entries[n].shape)
+            finally:
+                f.close()
+    except SafetensorsError as exc:
+        raise WeightsError(model_dir, [], [], [], [str(exc)]) from exc
+    return shapes
+
+
 def check_and_load(model_dir, specs: Iterable[TensorSpec], compute_dtype: torch.dtype,
                    device, may_be_unused: Iterable[str] = ()) -> Dict[str, torch.Tensor]:
     """Check the file(s) against ``specs`` and return ``{name: tensor on device}``.

@@ -156,8 +156,10 @@ def qk_norm_rope_store(qkv, n_heads, n_kv_heads, head_dim, q_norm_w, k_norm_w, e
 
 
 def paged_attention(q, n_heads, n_kv_heads, head_dim, k_pool, v_pool, row_pos, row_seg,
-                    block_tables, page_size, scale, window=0, **_unused):
+                    block_tables, page_size, scale, window=0, mods=None, **_unused):
     H, G, d = n_heads, n_kv_heads, head_dim
+    if mods is not None and not mods.active():
+        mods = None
     T = q.shape[0]
     out = torch.empty((T, H * d), dtype=F32)
     for t in range(T):
@@ -173,7 +175,16 @@ def paged_attention(q, n_heads, n_kv_heads, head_dim, k_pool, v_pool, row_pos, r
         for h in range(H):
             g = h // (H // G)
             sc = (keys[:, g, :] @ qt[h]) * scale
-            a = torch.softmax(sc, dim=0)
+            if mods is not None:
+                if mods.softcap > 0:
+                    sc = mods.softcap * torch.tanh(sc / mods.softcap)
+                if mods.distance_bias is not None:
+                    col = torch.clamp(p - idx, max=mods.distance_bias.shape[1] - 1)
+                    sc = sc + mods.distance_bias[h][col]
+            if mods is not None and mods.sink is not None:
+                a = torch.softmax(torch.cat([sc, mods.sink[h:h + 1]]), dim=0)[:-1]
+            else:
+                a = torch.softmax(sc, dim=0)
             out[t, h * d:(h + 1) * d] = a @ vals[:, g, :]
     return out.to(q.dtype)
 
@@ -366,6 +377,180 @@ def diff_combine(ctx, n_heads, n_kv_heads, vdim, head_size, lam, eps, gain):
 
 
 # ---- mixture of experts -----------------------------------------------------------------------
+# ---------------------------------------------------------------------------------------
+# the kernels of the output-norm arrangement, the scored and latent attention, the recurrences
+# with a matrix of state
+# ---------------------------------------------------------------------------------------
+def output_norm_add(resid, a, weight, eps, rows_dtype=None, scale_a=1.0, b=None, scale_b=1.0,
+                    add=True):
+    y = a.to(F32)
+    if y.dim() == 3:
+        acc = y[0].clone()
+        for part in y[1:]:
+            acc = acc + part
+        y = acc
+    y = y * scale_a
+    if b is not None:
+        y = y + scale_b * b.to(F32)
+    n = y * (1.0 / torch.sqrt((y * y).mean(dim=-1, keepdim=True) + eps)) * weight
+    if add:
+        resid.add_(n)
+    else:
+        resid.copy_(n)
+    return None if rows_dtype is None else resid.to(rows_dtype)
+
+
+def _store(k_pool, v_pool, keys, vals, row_pos, row_seg, block_tables, page_size):
+    for t in range(keys.shape[0]):
+        p = int(row_pos[t])
+        page = int(block_tables[int(row_seg[t]), p // page_size])
+        assert page >= 0, "a row is stored into a page that was given back"
+        k_pool[page, :, p % page_size, :] = keys[t].to(k_pool.dtype)
+        v_pool[page, :, :, p % page_size] = vals[t].to(v_pool.dtype)
+
+
+def projection_norm_store(proj, n_heads, n_kv_heads, dim, vdim, head_size, q_norm_w, k_norm_w, eps,
+                          temp_coef, temp_every, k_pool, v_pool, row_pos, row_seg, block_tables,
+                          page_size, store_kv=True):
+    H, G, d, dv, D = n_heads, n_kv_heads, dim, vdim, head_size
+    T = proj.shape[0]
+    p = proj.to(F32)
+    q, k, v = p[:, :H * d], p[:, H * d:(H + G) * d], p[:, (H + G) * d:(H + G) * d + G * dv]
+    if q_norm_w is not None:
+        q = q / torch.sqrt((q * q).mean(-1, keepdim=True) + eps) * q_norm_w
+    if k_norm_w is not None:
+        k = k / torch.sqrt((k * k).mean(-1, keepdim=True) + eps) * k_norm_w
+    if temp_coef:
+        steps = torch.div(row_pos.long() + 1, temp_every, rounding_mode="floor")
+        q = q * (1.0 + temp_coef * torch.log(steps.to(F32) + 1.0))[:, None]
+    qo = torch.zeros((T, H, D), dtype=F32)
+    qo[:, :, :d] = q.reshape(T, H, d)
+    if store_kv:
+        ko, vo = torch.zeros((T, G, D), dtype=F32), torch.zeros((T, G, D), dtype=F32)
+        ko[:, :, :d] = k.reshape(T, G, d)
+        vo[:, :, :dv] = v.reshape(T, G, dv)
+        _store(k_pool, v_pool, ko, vo, row_pos, row_seg, block_tables, page_size)
+    return qo.reshape(T, H * D).to(proj.dtype)
+
+
+def _rotate(x, pos, cos, sin, rot_dims, rot_mode):
+    if rot_mode == ROT_NONE or not rot_dims:
+        return x
+    half = rot_dims // 2
+    shape = [x.shape[0]] + [1] * (x.dim() - 2) + [half]
+    c, s = cos[pos].reshape(shape), sin[pos].reshape(shape)
+    y = x.clone()
+    if rot_mode == ROT_HALF:
+        a, b = x[..., :half], x[..., half:rot_dims]
+        y[..., :half] = a * c - b * s
+        y[..., half:rot_dims] = b * c + a * s
+    else:
+        a, b = x[..., 0:rot_dims:2], x[..., 1:rot_dims:2]
+        y[..., 0:rot_dims:2] = a * c - b * s
+        y[..., 1:rot_dims:2] = b * c + a * s
+    return y
+
+
+def latent_store(q, kv, n_heads, dim, rot_dim, rank, head_size, c_norm_w, eps, cos, sin, rot_dims,
+                 rot_mode, k_pool, v_pool, row_pos, row_seg, block_tables, page_size):
+    H, d, rot, r, D = n_heads, dim, rot_dim, rank, head_size
+    T = q.shape[0]
+    pos = row_pos.long()
+    kvf = kv.to(F32)
+    c = kvf[:, :r]
+    c = c / torch.sqrt((c * c).mean(-1, keepdim=True) + eps) * c_norm_w
+    key = torch.zeros((T, 1, D), dtype=F32)
+    key[:, 0, :r] = c
+    key[:, 0, r:r + rot] = _rotate(kvf[:, r:r + rot], pos, cos, sin, rot_dims, rot_mode)
+    val = torch.zeros((T, 1, D), dtype=F32)
+    val[:, 0, :r] = c
+    _store(k_pool, v_pool, key, val, row_pos, row_seg, block_tables, page_size)
+    out = torch.zeros((T, H, D), dtype=F32)
+    qr = q[:, :H * (d + rot)].to(F32).reshape(T, H, d + rot)[:, :, d:]
+    out[:, :, r:r + rot] = _rotate(qr, pos, cos, sin, rot_dims, rot_mode)
+    return out.reshape(T, H * D).to(q.dtype)
+
+
+def headwise_linear(x, x_head_stride, weight, out=None, out_head_stride=None):
+    H, n_out, n_in = weight.shape
+    T = x.shape[0]
+    if out is None:
+        out = torch.empty((T, H * n_out), dtype=x.dtype)
+        out_head_stride = n_out
+    for h in range(H):
+        xi = x[:, h * x_head_stride:h * x_head_stride + n_in].to(F32)
+        out[:, h * out_head_stride:h * out_head_stride + n_out] = (
+            xi @ weight[h].to(F32).T).to(out.dtype)
+    return out
+
+
+CONV_SILU_MAX_TAPS = 17
+GATE_SILU, GATE_SIGMOID = 0, 1
+
+
+def conv_silu(x, taps, state, row_pos, row_seg, seg_start, seg_pos0, seg_slot):
+    C, n = taps.shape
+    xf = x[:, :C].to(F32)
+    out = torch.empty((x.shape[0], C), dtype=F32)
+    for s in range(seg_slot.shape[0]):
+        t0, t1, slot = int(seg_start[s]), int(seg_start[s + 1]), int(seg_slot[s])
+        hist = torch.zeros((n - 1, C)) if int(seg_pos0[s]) == 0 else state[slot].clone()
+        seq = torch.cat([hist, xf[t0:t1]], dim=0)
+        for i in range(t1 - t0):
+            acc = torch.zeros(C)
+            for j in range(n):
+                acc = acc + taps[:, j] * seq[i + j]
+            out[t0 + i] = acc * torch.sigmoid(acc)
+        if n > 1:
+            state[slot] = seq[-(n - 1):]
+    return out.to(x.dtype)
+
+
+def matrix_state_recurrence(q, k, v, z, n_heads, n_qk_heads, dim, vdim, rate, z_bias, z_sign,
+                            q_scale, state, seg_start, seg_pos0, seg_slot, beta=None,
+                            unit_qk=False, unit_eps=1e-6):
+    H, Hk, d, dv = n_heads, n_qk_heads, dim, vdim
+    T = q.shape[0]
+    qf = q[:, :Hk * d].to(F32).reshape(T, Hk, d)
+    kf = k[:, :Hk * d].to(F32).reshape(T, Hk, d)
+    if unit_qk:
+        qf = qf / torch.sqrt((qf * qf).sum(-1, keepdim=True) + unit_eps)
+        kf = kf / torch.sqrt((kf * kf).sum(-1, keepdim=True) + unit_eps)
+    qf = (qf * q_scale).repeat_interleave(H // Hk, dim=1)
+    kf = kf.repeat_interleave(H // Hk, dim=1)
+    vf = v[:, :H * dv].to(F32).reshape(T, H, dv)
+    zz = z[:, :H * d].to(F32)
+    if z_bias is not None:
+        zz = zz + z_bias
+    a = torch.exp(-rate[:, None] * torch.nn.functional.softplus(z_sign * zz.reshape(T, H, d)))
+    b = torch.sigmoid(beta[:, :H].to(F32)) if beta is not None else None
+    out = torch.empty((T, H, dv), dtype=F32)
+    for s in range(seg_slot.shape[0]):
+        t0, t1, slot = int(seg_start[s]), int(seg_start[s + 1]), int(seg_slot[s])
+        S = torch.zeros((H, d, dv)) if int(seg_pos0[s]) == 0 else state[slot].clone()
+        for t in range(t0, t1):
+            S = a[t][:, :, None] * S
+            if b is not None:
+                u = b[t][:, None] * (vf[t] - torch.einsum("hdv,hd->hv", S, kf[t]))
+            else:
+                u = vf[t]
+            S = S + kf[t][:, :, None] * u[:, None, :]
+            out[t] = torch.einsum("hdv,hd->hv", S, qf[t])
+        state[slot] = S
+    return out.reshape(T, H * dv)
+
+
+def head_norm_gate(o, weight, eps, gate, gate_kind, n_heads, vdim, out_dtype):
+    H, dv = n_heads, vdim
+    T = o.shape[0]
+    x = o.reshape(T, H, dv)
+    x = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * weight
+    g = gate[:, :H * dv].to(F32).reshape(T, H, dv)
+    g = g * torch.sigmoid(g) if gate_kind == GATE_SILU else torch.sigmoid(g)
+    return (x * g).reshape(T, H * dv).to(out_dtype)
+
+
+
 class _Plan:
     def __init__(self, experts):
         self.experts = experts
@@ -408,6 +593,8 @@ def moe_combine(y, weights, plan):
 
 ALL = ["add_group_rmsnorm", "add_group_rmsnorm_canon_step", "canon_conv", "scale_add_positions", "glu", "mingru_scan", "diff_store",
        "diff_combine", "moe_route", "moe_plan", "moe_experts_gated", "moe_experts_down", "moe_combine",
+       "output_norm_add", "projection_norm_store", "latent_store", "headwise_linear", "conv_silu",
+       "matrix_state_recurrence", "head_norm_gate",
        "embed_rows", "add_rmsnorm", "add_residual", "sum_partial_sums", "swiglu", "cast", "linear", "linear_swiglu",
        "interleave_gate_up", "shortconv", "linear_shortconv_step",
        "qk_norm_rope_store", "paged_attention", "sample_rows", "sample_filtered",
