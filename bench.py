@@ -104,7 +104,11 @@ def run_workload(key, dtype, device, repeat_penalty=1.0):
 # --compare: the Dapipel decoder beside the LFM2 shape of the same width, depth, attention layers
 # and feed-forward width (config/shapes.py), both with random weights
 COMPARISONS = {"w1024": ("dapipel-w1024", "lfm2-like-w1024"),
-               "w2048": ("dapipel-w2048", "lfm2-like-w2048")}
+               "w2048": ("dapipel-w2048", "lfm2-like-w2048"),
+               # the Dukolorn decoder beside the same LFM2 shapes (its closest relative: a hybrid
+               # of recurrent and attention layers with SiLU-gated dense feed-forwards)
+               "dukolorn-w1024": ("dukolorn-w1024", "lfm2-like-w1024"),
+               "dukolorn-w2048": ("dukolorn-w2048", "lfm2-like-w2048")}
 
 
 def stage_table(runner, entries_of, reps):
@@ -191,8 +195,8 @@ def run_comparison(keys, args):
                                       min(args.context, 2048), args.steps, args.warmup,
                                       args.page_size) for n in (new, old)]
         print(f"bench.py: {key} done", file=sys.stderr, flush=True)
-    print(json.dumps({"metric": "prefill and decode tok/s, Dapipel beside the LFM2 shape of equal "
-                                "size", "unit": "tok/s", "n_gpus": 1, "dtype": args.dtype,
+    print(json.dumps({"metric": "prefill and decode tok/s, a decoder beside the LFM2 shape of "
+                                "equal size", "unit": "tok/s", "n_gpus": 1, "dtype": args.dtype,
                       "data": "synthetic", "prefill_tokens": args.prefill_tokens,
                       "batch": args.batch, "context": min(args.context, 2048),
                       "steps": args.steps, "warmup": args.warmup, "sizes": results}))
@@ -563,12 +567,14 @@ def main() -> int:
                     help="serving workloads: a repeat penalty over the last 64 tokens before "
                          "the greedy choice (1: none)")
     ap.add_argument("--compare", default="", metavar="SIZES",
-                    help="instead of the headline run: prompt and decode steps of the Dapipel "
-                         "decoder beside the LFM2 shape of equal size, at these sizes (comma "
+                    help="instead of the headline run: prompt and decode steps of the Dapipel or "
+                         "Dukolorn decoder beside the LFM2 shape of equal size, at these sizes (comma "
                          "separated: " + ", ".join(sorted(COMPARISONS)) + "; 'all')")
     args = ap.parse_args()
     if args.compare:
-        keys = sorted(COMPARISONS) if args.compare == "all" else args.compare.split(",")
+        keys = (sorted(k for k in COMPARISONS if k.startswith("w")) if args.compare == "all"
+                else sorted(k for k in COMPARISONS if k.startswith("dukolorn"))
+                if args.compare == "dukolorn" else args.compare.split(","))
         for k in keys:
             if k not in COMPARISONS:
                 print(f"bench.py: no comparison {k!r}; known: {', '.join(sorted(COMPARISONS))}")

@@ -101,6 +101,56 @@ SHAPES.update({
 })
 
 
+def _dukolorn(width, mixers, heads, kv_heads, dim, r_heads, r_dim, r_vdim, l_heads, l_dim, l_rot,
+              l_vdim, l_rank, window, d_heads, d_qk_heads, d_dim, d_vdim, ff, vocab=65536,
+              rank=32, buckets=64, bias_max=512.0) -> dict:
+    """Layers by letter: "p" a scored softmax attention beside a gated linear attention, "l" a
+    latent attention under a sliding window, "d" the gated delta rule (without feed-forward, as
+    the design's own models have it); dense feed-forwards of ``ff`` elsewhere."""
+    layers = []
+    for kind in mixers:
+        if kind == "p":
+            left = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": dim,
+                    "scale": dim ** -0.5, "softcap": 50.0, "bias_max": bias_max,
+                    "buckets": buckets, "q_temp": {"coef": 0.1, "every": 256}}
+            right = {"heads": r_heads, "dim": r_dim, "vdim": r_vdim, "tau": 8.0,
+                     "decay_rank": rank}
+            layers.append({"type": "parallel", "mlp": {"kind": "dense", "ff": ff},
+                           "mixer": {"left": left, "right": right, "left_scale": 1.0,
+                                     "right_scale": 1.0}})
+        elif kind == "l":
+            layers.append({"type": "latent_attention", "mlp": {"kind": "dense", "ff": ff},
+                           "mixer": {"heads": l_heads, "dim": l_dim, "rot_dim": l_rot,
+                                     "vdim": l_vdim, "kv_rank": l_rank,
+                                     "scale": (l_dim + l_rot) ** -0.5,
+                                     "rot": {"base": 10000.0, "dims": l_rot},
+                                     "mask": {"size": window}}})
+        else:
+            layers.append({"type": "channel_delta", "mlp": None,
+                           "mixer": {"heads": d_heads, "kv_heads": d_qk_heads, "dim": d_dim,
+                                     "vdim": d_vdim, "conv": 4, "decay_rank": rank,
+                                     "gate_rank": rank}})
+    return {"architecture": "Dukolorn", "vocab": vocab, "width": width, "norm": {"eps": 1e-5},
+            "logit_scale": 1.0, "layers": layers}
+
+
+SHAPES.update({
+    # eight layers at a width of 1024 in the order pair, latent, latent, delta rule, twice: 16
+    # heads of 64 on 4 kv heads beside 8 recurrent heads of 64 x 64; latent attention with 16
+    # heads of 64 + 32 rotated places on a latent of 224 under a window of 1024; the delta rule
+    # with 16 heads of 64 x 64 on 4 q/k heads; feed-forward 4608
+    "dukolorn-w1024": _dukolorn(1024, "plldplld", 16, 4, 64, 8, 64, 64, 16, 64, 32, 64, 224, 1024,
+                                16, 4, 64, 64, 4608),
+    # the same at a width of 2048: 32 heads on 8 kv heads, recurrent heads of 64 x 128, 16 latent
+    # heads of 128 + 64 on a latent of 192 under a window of 2048, feed-forward 8192
+    "dukolorn-w2048": _dukolorn(2048, "plldplld", 32, 8, 64, 16, 64, 128, 16, 128, 64, 128, 192,
+                                2048, 16, 4, 128, 128, 8192),
+    # a tiny one for smoke runs
+    "dukolorn-tiny": _dukolorn(64, "pld", 4, 2, 8, 2, 8, 16, 2, 8, 8, 16, 24, 24, 2, 1, 16, 8, 96,
+                               vocab=256, rank=4, buckets=8, bias_max=40.0),
+})
+
+
 def named_shape(name: str) -> dict:
     """A copy of the configuration called ``name`` (any case), or a ``KeyError`` naming them all."""
     key = name.strip().lower()

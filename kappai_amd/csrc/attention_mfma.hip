@@ -20,6 +20,7 @@
 // 623-666), online softmax as in its flash form (:386-413).
 #include "common.h"
 #include "no_alloc.h"
+#include "score_mods.h"
 #include <stdio.h>
 
 #ifndef HEAD_DIM
@@ -138,12 +139,15 @@ __device__ __forceinline__ u32x4_t load_k8(const bf16_t* __restrict__ k_pool,
 // longest chain of dependent work fourfold; their partial results meet in LDS
 #define P_NW (HEAD_DIM <= 128 ? 4 : 1)
 
+// MODS: the scores pass kappai_modified_score (a cap, a bias by distance) between the scaled
+// product and the softmax, and a sink may join the denominator (score_mods.h).
+template <bool MODS>
 __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ vt_pool, bf16_t* __restrict__ out, int out_stride,
     const int* __restrict__ q_tiles, const int* __restrict__ row_pos,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int ps, int window,
-    float scale) {
+    float scale, kappai_score_mods mods) {
   // later tiles of a segment have more keys: they are started first
   const int tile = gridDim.x - 1 - blockIdx.x, h = blockIdx.y;
   const int lane = threadIdx.x % WAVE;
@@ -176,7 +180,8 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
 #pragma unroll
     for (int v = 0; v < 16; ++v) o[mt][v] = 0.f;
   float m_run = -INFINITY, l_run = 0.f;
-  const float sc = scale * LOG2E;
+  // (with MODS the scores are scaled, worked on and brought to units of log 2 one by one)
+  const float sc = MODS ? 1.0f : scale * LOG2E;
 
   // A tile of 32 keys is "whole" when every row of the q tile sees all of its keys: then nothing
   // is masked, and addresses are a base that is the same for all lanes of a 16-key group (its
@@ -246,6 +251,13 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
     for (int ks = 0; ks < P_KS; ++ks)
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(kfr[buf][ks]), qf[ks], s, 0, 0, 0);
     // lane holds, for query `col`, keys kb + 8*(v/4) + 4*hh + v%4
+    if (MODS) {
+#pragma unroll
+      for (int v = 0; v < 16; ++v) {
+        const int key = kb + 8 * (v / 4) + 4 * hh + v % 4;
+        s[v] = kappai_modified_score(mods, s[v] * scale, h, my_pos - key) * LOG2E;
+      }
+    }
     float mloc = -INFINITY;
     if (whole(kb)) {
 #pragma unroll
@@ -335,6 +347,8 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
     l_run = sh_l[0][col];
 #pragma unroll
     for (int w = 1; w < P_NW; ++w) l_run += sh_l[w][col];
+    if (MODS && mods.sink != nullptr && M != -INFINITY)
+      l_run += fast_exp2(mods.sink[h] * LOG2E - M);
 #pragma unroll
     for (int mt = 0; mt < P_MT; ++mt)
 #pragma unroll
@@ -346,6 +360,8 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
       }
   }
   if (!row_ok) return;
+  if (MODS && P_NW == 1 && mods.sink != nullptr && m_run != -INFINITY)
+    l_run += fast_exp2(mods.sink[h] * LOG2E - m_run);
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
   bf16_t* orow = out + (size_t)(r0 + col) * out_stride + (size_t)h * HEAD_DIM;
 #pragma unroll
@@ -881,12 +897,13 @@ __device__ __forceinline__ void qk_norm_rotate(u32x4_t (&raw)[(HEAD_DIM + 31) / 
 // of the chunks c0 = first, first + stride, ... below k_end (D_KPW keys each), with a running
 // maximum and sum per column.  Leaves the unnormalised output in o (lane: column lane % 16, d
 // rows 16 mt + 4 (lane / 16) + v), the maximum (in units of log 2) in m_run, the sum in l_run.
-template <bool FUSABLE>
+template <bool FUSABLE, bool MODS = false>
 __device__ __forceinline__ void attn_decode_wave(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ vt_pool, const int* __restrict__ bt, int max_blocks, int t, int g,
     int H, int G, int ps, float scale, int lo, int hi, int first, int stride, int k_end,
-    f32x4_t (&o)[D_MT], float& m_run, float& l_run, const QkFuse& qk, int pos) {
+    f32x4_t (&o)[D_MT], float& m_run, float& l_run, const QkFuse& qk, int pos,
+    const kappai_score_mods* mods = nullptr) {
   const int lane = threadIdx.x % WAVE;
   const int rep = H / G;
   const int col = lane % 16, kg = lane / 16;
@@ -1033,7 +1050,11 @@ __device__ __forceinline__ void attn_decode_wave(
         for (int v = 0; v < 4; ++v) {
           const int key = kb + 8 * kg + 4 * tt + v;
           const bool ok = key >= lo && key <= hi;
-          s[tt][v] = ok ? s[tt][v] * sc : -INFINITY;
+          if (MODS)
+            s[tt][v] = ok ? kappai_modified_score(*mods, s[tt][v] * scale, h, pos - key) * LOG2E
+                          : -INFINITY;
+          else
+            s[tt][v] = ok ? s[tt][v] * sc : -INFINITY;
           mloc = fmaxf(mloc, s[tt][v]);
         }
       mloc = fmaxf(mloc, __shfl_xor(mloc, 16, WAVE));
@@ -1135,13 +1156,14 @@ __device__ __forceinline__ int step_keys_per_split(const int* __restrict__ row_p
 // halve the waves a SIMD holds for the steps that do not use it)
 // (PLAN: the keys per split come from step_keys_per_split, else they are the caller's: a kernel of
 // its own, because the rule's code costs half a microsecond even where it is skipped)
-template <bool FUSED, bool PLAN>
+template <bool FUSED, bool PLAN, bool MODS = false>
 __global__ __launch_bounds__(64) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ vt_pool, float* __restrict__ part_o, float* __restrict__ part_ml,
     const int* __restrict__ row_pos, const int* __restrict__ row_seg,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int ps, int window,
-    float scale, int keys_per_split, int n_splits, QkFuse qk, const int* __restrict__ row_ids) {
+    float scale, int keys_per_split, int n_splits, QkFuse qk, const int* __restrict__ row_ids,
+    kappai_score_mods mods) {
   // (row_ids: the kernel's rows are these rows of the step, partial results are kept by their
   // place in the list)
   // Blocks go to the CUs in the order of their numbers, the row's number fastest: with a number
@@ -1168,8 +1190,9 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
   const size_t pbase = ((size_t)ti * H + h) * n_splits + split;
   f32x4_t o[D_MT];
   float m_run, l_run;
-  attn_decode_wave<FUSED>(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale, lo,
-                          k_end - 1, k_begin, D_KPW, k_end, o, m_run, l_run, qk, pos);
+  attn_decode_wave<FUSED, MODS>(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale,
+                                lo, k_end - 1, k_begin, D_KPW, k_end, o, m_run, l_run, qk, pos,
+                                &mods);
   if (!head_ok) return;
   if (kg == 0) {
     part_ml[2 * pbase] = m_run;
@@ -1190,12 +1213,13 @@ __global__ __launch_bounds__(64) void attn_decode_kernel(
 // keys depends on the row's own position and on the number of waves only.  For batches with
 // (rows x kv heads) enough to fill the chip, or contexts short enough for one block.
 // LDS: sh_o [NW][rep][HEAD_DIM], then sh_m [NW][16], sh_l [NW][16] (floats).
+template <bool MODS>
 __global__ __launch_bounds__(D_BLOCK_MAX_WAVES * WAVE) void attn_decode_block_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
     const bf16_t* __restrict__ vt_pool, bf16_t* __restrict__ out, int out_stride,
     const int* __restrict__ row_pos, const int* __restrict__ row_seg,
     const int* __restrict__ block_tables, int max_blocks, int H, int G, int ps, int window,
-    float scale) {
+    float scale, kappai_score_mods mods) {
   extern __shared__ float sh_dec[];
   const int t = blockIdx.x, g = blockIdx.y;
   const int lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE, NW = blockDim.x / WAVE;
@@ -1210,9 +1234,9 @@ __global__ __launch_bounds__(D_BLOCK_MAX_WAVES * WAVE) void attn_decode_block_ke
   float m_run, l_run;
   // (without the prologue: eight waves a block leave no registers for it, and every wave would
   // do it again)
-  attn_decode_wave<false>(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale, lo,
-                          pos, k_begin + wave * D_KPW, NW * D_KPW, k_end, o, m_run, l_run,
-                          QkFuse{}, pos);
+  attn_decode_wave<false, MODS>(q, q_stride, k_pool, vt_pool, bt, max_blocks, t, g, H, G, ps, scale,
+                                lo, pos, k_begin + wave * D_KPW, NW * D_KPW, k_end, o, m_run,
+                                l_run, QkFuse{}, pos, &mods);
   float* sh_o = sh_dec;
   float* sh_m = sh_dec + (size_t)NW * rep * HEAD_DIM;
   float* sh_l = sh_m + NW * 16;
@@ -1239,6 +1263,8 @@ __global__ __launch_bounds__(D_BLOCK_MAX_WAVES * WAVE) void attn_decode_block_ke
       L += sh_l[w * 16 + c] * wgt;
       acc = fmaf(sh_o[((size_t)w * rep + c) * HEAD_DIM + e], wgt, acc);
     }
+    if (MODS && mods.sink != nullptr && M != -INFINITY)
+      L += fast_exp2(mods.sink[g * rep + c] * LOG2E - M);
     const float inv = L > 0.f ? 1.0f / L : 0.f;
     out[(size_t)t * out_stride + (size_t)(g * rep + c) * HEAD_DIM + e] = f32_to_bf16(acc * inv);
   }
@@ -1254,7 +1280,7 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
     const float* __restrict__ part_o, const float* __restrict__ part_ml,
     bf16_t* __restrict__ out, int out_stride, int H, int splits_stride,
     const int* __restrict__ row_ids, const int* __restrict__ row_pos, int window, int G,
-    int kps_min, int planned) {
+    int kps_min, int planned, const float* __restrict__ sink) {
   constexpr int NPL = (HEAD_DIM + WAVE - 1) / WAVE;
   __shared__ float sh_acc[MERGE_WAVES][NPL * WAVE];
   __shared__ float sh_l[MERGE_WAVES];
@@ -1329,6 +1355,7 @@ __global__ __launch_bounds__(MERGE_WAVES * WAVE) void attn_merge_kernel(
   __syncthreads();
   if (wave != 0) return;
   L = (sh_l[0] + sh_l[1]) + (sh_l[2] + sh_l[3]);
+  if (sink != nullptr && M != -INFINITY) L += fast_exp2(sink[h] * LOG2E - M);   // (sink: a logit)
   const float inv = L > 0.f ? 1.0f / L : 0.f;
   bf16_t* dst = out + (size_t)t * out_stride + (size_t)h * HEAD_DIM;
 #pragma unroll
@@ -1354,23 +1381,42 @@ extern "C" int kappai_attn_decode_block_waves(int rep) {
 
 // Decode attention with the keys of a row split over the `n_waves` waves of one block per (row, kv
 // head); no workspace, no second kernel.
-extern "C" int kappai_attn_decode_block(const void* q, int q_stride, const void* k_pool,
-                                        const void* vt_pool, void* out, int out_stride,
-                                        const int* row_pos, const int* row_seg,
-                                        const int* block_tables, int max_blocks, int T, int H,
-                                        int G, int ps, int window, float scale, int n_waves,
-                                        hipStream_t stream) {
+// `mods` (may be null): a cap on the scores, a bias by distance, a sink (score_mods.h).
+extern "C" int kappai_attn_decode_block_scored(const void* q, int q_stride, const void* k_pool,
+                                               const void* vt_pool, void* out, int out_stride,
+                                               const int* row_pos, const int* row_seg,
+                                               const int* block_tables, int max_blocks, int T,
+                                               int H, int G, int ps, int window, float scale,
+                                               int n_waves, const kappai_score_mods* mods,
+                                               hipStream_t stream) {
   if (T <= 0) return 0;
   if (ps % 16 || G < 1 || H % G || H / G > 16 || G > 65535 || (q_stride % 8) || n_waves < 1 ||
       n_waves > kappai_attn_decode_block_waves(H / G))
     return (int)hipErrorInvalidValue;
   const int rep = H / G;
   const size_t lds = (size_t)n_waves * (rep * HEAD_DIM + 32) * sizeof(float);
-  hipLaunchKernelGGL(attn_decode_block_kernel, dim3(T, G), dim3(n_waves * WAVE), lds, stream,
-                     (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
-                     (bf16_t*)out, out_stride, row_pos, row_seg, block_tables, max_blocks, H, G, ps,
-                     window, scale);
+  if (kappai_mods_on(mods))
+    hipLaunchKernelGGL(attn_decode_block_kernel<true>, dim3(T, G), dim3(n_waves * WAVE), lds,
+                       stream, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool,
+                       (const bf16_t*)vt_pool, (bf16_t*)out, out_stride, row_pos, row_seg,
+                       block_tables, max_blocks, H, G, ps, window, scale, *mods);
+  else
+    hipLaunchKernelGGL(attn_decode_block_kernel<false>, dim3(T, G), dim3(n_waves * WAVE), lds,
+                       stream, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool,
+                       (const bf16_t*)vt_pool, (bf16_t*)out, out_stride, row_pos, row_seg,
+                       block_tables, max_blocks, H, G, ps, window, scale, kappai_score_mods{0.f, nullptr, 0, nullptr});
   KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int kappai_attn_decode_block(const void* q, int q_stride, const void* k_pool,
+                                        const void* vt_pool, void* out, int out_stride,
+                                        const int* row_pos, const int* row_seg,
+                                        const int* block_tables, int max_blocks, int T, int H,
+                                        int G, int ps, int window, float scale, int n_waves,
+                                        hipStream_t stream) {
+  return kappai_attn_decode_block_scored(q, q_stride, k_pool, vt_pool, out, out_stride, row_pos,
+                                         row_seg, block_tables, max_blocks, T, H, G, ps, window,
+                                         scale, n_waves, nullptr, stream);
 }
 
 // 1 when the decode kernel of this head size that splits the keys over blocks can do the per-head
@@ -1396,12 +1442,24 @@ extern "C" int kappai_attn_head_dim(void) { return HEAD_DIM; }
 
 // variant: 0 = chosen by shape, 1 = one block per (tile, head), 2 = key tiles shared by four
 // query heads of a kv head (head sizes 64 and 128, a multiple of four heads per kv head).
-extern "C" int kappai_attn_prefill(const void* q, int q_stride, const void* k_pool,
-                                   const void* vt_pool, void* out, int out_stride,
-                                   const int* q_tiles, int n_tiles, const int* row_pos,
-                                   const int* block_tables, int max_blocks, int H, int G, int ps,
-                                   int window, float scale, int variant, hipStream_t stream) {
+// `mods` (may be null; score_mods.h): with them the kernel of one block a (tile, head) runs.
+extern "C" int kappai_attn_prefill_scored(const void* q, int q_stride, const void* k_pool,
+                                          const void* vt_pool, void* out, int out_stride,
+                                          const int* q_tiles, int n_tiles, const int* row_pos,
+                                          const int* block_tables, int max_blocks, int H, int G,
+                                          int ps, int window, float scale, int variant,
+                                          const kappai_score_mods* mods, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
+  if (kappai_mods_on(mods)) {
+    if (ps % 16 || G < 1 || H % G || H > 65535 || (q_stride % 8) || (out_stride % 4) ||
+        variant == 2 || (mods->dist_bias != nullptr && mods->dist_cols < 1))
+      return (int)hipErrorInvalidValue;
+    hipLaunchKernelGGL(attn_prefill_kernel<true>, dim3(n_tiles, H), dim3(P_NW * WAVE), 0, stream,
+                       (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
+                       (bf16_t*)out, out_stride, q_tiles, row_pos, block_tables, max_blocks, H, G,
+                       ps, window, scale, *mods);
+    KAPPAI_RETURN_LAUNCH_STATUS();
+  }
   if (ps % 16 || G < 1 || H % G || H > 65535 || (q_stride % 8) || (out_stride % 4))
     return (int)hipErrorInvalidValue;
   const int rep = H / G;
@@ -1419,11 +1477,21 @@ extern "C" int kappai_attn_prefill(const void* q, int q_stride, const void* k_po
     KAPPAI_RETURN_LAUNCH_STATUS();
   }
 #endif
-  hipLaunchKernelGGL(attn_prefill_kernel, dim3(n_tiles, H), dim3(P_NW * WAVE), 0, stream,
+  hipLaunchKernelGGL(attn_prefill_kernel<false>, dim3(n_tiles, H), dim3(P_NW * WAVE), 0, stream,
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
                      (bf16_t*)out, out_stride, q_tiles, row_pos, block_tables, max_blocks, H, G,
-                     ps, window, scale);
+                     ps, window, scale, kappai_score_mods{0.f, nullptr, 0, nullptr});
   KAPPAI_RETURN_LAUNCH_STATUS();
+}
+
+extern "C" int kappai_attn_prefill(const void* q, int q_stride, const void* k_pool,
+                                   const void* vt_pool, void* out, int out_stride,
+                                   const int* q_tiles, int n_tiles, const int* row_pos,
+                                   const int* block_tables, int max_blocks, int H, int G, int ps,
+                                   int window, float scale, int variant, hipStream_t stream) {
+  return kappai_attn_prefill_scored(q, q_stride, k_pool, vt_pool, out, out_stride, q_tiles,
+                                    n_tiles, row_pos, block_tables, max_blocks, H, G, ps, window,
+                                    scale, variant, nullptr, stream);
 }
 
 static int launch_decode(const void* q, int q_stride, const void* k_pool, const void* vt_pool,
@@ -1431,8 +1499,11 @@ static int launch_decode(const void* q, int q_stride, const void* k_pool, const 
                          const int* row_pos, const int* row_seg, const int* block_tables,
                          int max_blocks, int T, int H, int G, int ps, int window, float scale,
                          int keys_per_split, int n_splits, const QkFuse& qk, const int* row_ids,
-                         hipStream_t stream) {
+                         hipStream_t stream, const kappai_score_mods* mods = nullptr) {
   if (T <= 0) return 0;
+  const bool scored = kappai_mods_on(mods);
+  if (scored && qk.on) return (int)hipErrorInvalidValue;
+  const kappai_score_mods m = scored ? *mods : kappai_score_mods{0.f, nullptr, 0, nullptr};
   if (ps % 16 || G < 1 || H % G || H / G > 16 || G > 65535 || n_splits < 1 || n_splits > 65535 ||
       keys_per_split < D_KPW || keys_per_split % D_KPW || (q_stride % 8))
     return (int)hipErrorInvalidValue;
@@ -1440,18 +1511,21 @@ static int launch_decode(const void* q, int q_stride, const void* k_pool, const 
   // aimed at (else they could not ask for longer splits than the grid's own), and not in the form
   // with the prologue, which runs for a few rows and has no registers to spare.
   const bool plan = !qk.on && (long long)T * G * n_splits > D_TARGET_WAVES;
-#define KAPPAI_DECODE(FUSED, PLAN)                                                               \
-  hipLaunchKernelGGL((attn_decode_kernel<FUSED, PLAN>), dim3(T, G, n_splits), dim3(WAVE), 0,     \
-                     stream, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool,                  \
+#define KAPPAI_DECODE(FUSED, PLAN, MODS)                                                         \
+  hipLaunchKernelGGL((attn_decode_kernel<FUSED, PLAN, MODS>), dim3(T, G, n_splits), dim3(WAVE),  \
+                     0, stream, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool,               \
                      (const bf16_t*)vt_pool, part_o, part_ml, row_pos, row_seg, block_tables,    \
-                     max_blocks, H, G, ps, window, scale, keys_per_split, n_splits, qk, row_ids)
-  if (qk.on) KAPPAI_DECODE(true, false);
-  else if (plan) KAPPAI_DECODE(false, true);
-  else KAPPAI_DECODE(false, false);
+                     max_blocks, H, G, ps, window, scale, keys_per_split, n_splits, qk, row_ids, \
+                     m)
+  if (qk.on) KAPPAI_DECODE(true, false, false);
+  else if (scored && plan) KAPPAI_DECODE(false, true, true);
+  else if (scored) KAPPAI_DECODE(false, false, true);
+  else if (plan) KAPPAI_DECODE(false, true, false);
+  else KAPPAI_DECODE(false, false, false);
 #undef KAPPAI_DECODE
   hipLaunchKernelGGL(attn_merge_kernel, dim3(T, H), dim3(MERGE_WAVES * WAVE), 0, stream,
                      (const float*)part_o, (const float*)part_ml, (bf16_t*)out, out_stride, H,
-                     n_splits, row_ids, row_pos, window, G, keys_per_split, plan ? 1 : 0);
+                     n_splits, row_ids, row_pos, window, G, keys_per_split, plan ? 1 : 0, m.sink);
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
@@ -1464,6 +1538,20 @@ extern "C" int kappai_attn_decode(const void* q, int q_stride, const void* k_poo
   return launch_decode(q, q_stride, k_pool, vt_pool, out, out_stride, part_o, part_ml, row_pos,
                        row_seg, block_tables, max_blocks, T, H, G, ps, window, scale,
                        keys_per_split, n_splits, QkFuse{}, nullptr, stream);
+}
+
+// kappai_attn_decode (row_ids null) or kappai_attn_decode_rows with `mods` (score_mods.h).
+extern "C" int kappai_attn_decode_scored(const void* q, int q_stride, const void* k_pool,
+                                         const void* vt_pool, void* out, int out_stride,
+                                         float* part_o, float* part_ml, const int* row_ids,
+                                         const int* row_pos, const int* row_seg,
+                                         const int* block_tables, int max_blocks, int T, int H,
+                                         int G, int ps, int window, float scale,
+                                         int keys_per_split, int n_splits,
+                                         const kappai_score_mods* mods, hipStream_t stream) {
+  return launch_decode(q, q_stride, k_pool, vt_pool, out, out_stride, part_o, part_ml, row_pos,
+                       row_seg, block_tables, max_blocks, T, H, G, ps, window, scale,
+                       keys_per_split, n_splits, QkFuse{}, row_ids, stream, mods);
 }
 
 // kappai_attn_decode for some rows of a step: row_ids [T] names them (rows of q, row_pos, row_seg

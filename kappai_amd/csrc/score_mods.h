@@ -14,11 +14,15 @@ struct kappai_score_mods {
   const float* sink;
 };
 
+__host__ __device__ __forceinline__ bool kappai_mods_on(const kappai_score_mods* m) {
+  return m != nullptr && (m->softcap > 0.f || m->dist_bias != nullptr || m->sink != nullptr);
+}
+
 // `s` is the scaled dot product; the result is what the softmax sees (natural-logarithm units).
 __device__ __forceinline__ float kappai_modified_score(const kappai_score_mods& m, float s, int h,
                                                        int dist) {
   if (m.softcap > 0.f) s = m.softcap * tanhf(s / m.softcap);
   if (m.dist_bias != nullptr)
-    s += m.dist_bias[(size_t)h * m.dist_cols + min(dist, m.dist_cols - 1)];
+    s += m.dist_bias[(size_t)h * m.dist_cols + max(0, min(dist, m.dist_cols - 1))];
   return s;
 }

@@ -941,8 +941,6 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
             kernel = "prefill"
         else:
             kernel = "rows"
-    if mods is not None:
-        kernel = "rows"            # (the only kernel that knows them yet)
     if kernel == "rows":
         check(library("attention").kappai_paged_attention_rows_scored(
             _ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
@@ -958,11 +956,11 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
     if kernel == "prefill":
         _gpu("q_tiles", q_tiles, I32)
         _need(q_tiles.dim() == 2 and q_tiles.shape[1] == 4, "q_tiles must be [tiles, 4]")
-        check(lib.kappai_attn_prefill(
+        check(lib.kappai_attn_prefill_scored(
             _ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
             _ptr(q_tiles), _c_int(q_tiles.shape[0]), _ptr(row_pos), _ptr(block_tables),
             _c_int(block_tables.shape[1]), _c_int(H), _c_int(G), _c_int(page_size),
-            _c_int(window or 0), _c_float(scale), _c_int(prefill_variant), _stream()),
+            _c_int(window or 0), _c_float(scale), _c_int(prefill_variant), mods_ref, _stream()),
             "attn_prefill")
         if lone_rows is not None:
             _gpu("lone_rows", lone_rows, I32)
@@ -970,13 +968,16 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
                   "paged_attention: rows left out of the tiles need the decode kernel (at most 16 "
                   "query heads a kv head) and their largest position")
             _decode_split(lib, q, H, G, d, k_pool, v_pool, row_pos, row_seg, block_tables,
-                          page_size, scale, window, max_lone_position, out, lone_rows)
+                          page_size, scale, window, max_lone_position, out, lone_rows,
+                          mods_ref=mods_ref)
         return out
     _need(kernel in ("decode", "decode-block", "decode-split"),
           lambda: f"unknown attention kernel {kernel!r}")
     _need(H // G <= 16, "the decode kernel takes at most 16 query heads per kv head")
     _need(max_position is not None, "the decode kernel needs the batch's largest position")
     qk_args = ()
+    _need(qk is None or mods is None, "paged_attention: the decode kernels do either the norm and "
+          "the rotation themselves or work on the scores, not both")
     if qk is not None:
         _need(bool(lib.kappai_attn_decode_takes_qk()),
               lambda: f"the decode kernels of head size {d} do not take the norm and the rotation")
@@ -1004,14 +1005,14 @@ def paged_attention(q: torch.Tensor, n_heads: int, n_kv_heads: int, head_dim: in
         _need(block_waves > 0, "too many query heads a kv head for the block form")
         _need(qk is None, "the decode kernel that keeps a row's keys in one block takes q ready "
                           "made and the keys stored")
-        check(lib.kappai_attn_decode_block(
+        check(lib.kappai_attn_decode_block_scored(
             _ptr(q), _c_int(q.stride(0)), _ptr(k_pool), _ptr(v_pool), _ptr(out), _c_int(H * d),
             _ptr(row_pos), _ptr(row_seg), _ptr(block_tables), _c_int(block_tables.shape[1]),
             _c_int(T), _c_int(H), _c_int(G), _c_int(page_size), _c_int(window or 0),
-            _c_float(scale), _c_int(block_waves), _stream()), "attn_decode_block")
+            _c_float(scale), _c_int(block_waves), mods_ref, _stream()), "attn_decode_block")
         return out
     _decode_split(lib, q, H, G, d, k_pool, v_pool, row_pos, row_seg, block_tables, page_size, scale,
-                  window, max_position, out, None, qk_args)
+                  window, max_position, out, None, qk_args, mods_ref=mods_ref)
     return out
 
 
@@ -1026,7 +1027,7 @@ def decode_splits(keys_per_wave: int, rows: int, n_kv_heads: int, n_keys: int):
 
 
 def _decode_split(lib, q, H, G, d, k_pool, v_pool, row_pos, row_seg, block_tables, page_size, scale,
-                  window, max_position, out, row_ids, qk_args=()):
+                  window, max_position, out, row_ids, qk_args=(), mods_ref=None):
     """The decode kernel that splits a row's keys over blocks, and its merge, for all rows or
     (``row_ids``) some of them."""
     T = q.shape[0] if row_ids is None else row_ids.shape[0]
@@ -1047,7 +1048,10 @@ def _decode_split(lib, q, H, G, d, k_pool, v_pool, row_pos, row_seg, block_table
     tail = (_ptr(row_pos), _ptr(row_seg), _ptr(block_tables), _c_int(block_tables.shape[1]),
             _c_int(T), _c_int(H), _c_int(G), _c_int(page_size), _c_int(window or 0),
             _c_float(scale), _c_int(keys_per_split), _c_int(n_splits))
-    if row_ids is not None:
+    if mods_ref is not None:
+        check(lib.kappai_attn_decode_scored(*head, _ptr(row_ids), *tail, mods_ref, _stream()),
+              "attn_decode_scored")
+    elif row_ids is not None:
         check(lib.kappai_attn_decode_rows(*head, _ptr(row_ids), *tail, _stream()),
               "attn_decode_rows")
     elif qk_args:

@@ -126,8 +126,10 @@ FP32_TOL = 2e-5
 
 def assert_matches_plain(got, model_dir, requests, dtype, what=""):
     """float32: every row within FP32_TOL.  bfloat16: against what rounding the same values to
-    bfloat16 costs the plain implementation itself: no row over six times its root mean square
-    row error and at most one row in fifty over three times."""
+    bfloat16 costs the plain implementation itself.  Its root mean square row error is the yard:
+    no row over six yards and at most one row in fifty over three, but for rows where the plain
+    implementation's own rounding error is that large too (a few rows are far more sensitive than
+    the rest; there a row may err by half as much again as the plain one)."""
     ref = plain_logits(model_dir, requests)
     errs = row_errors(got, ref)
     worst = max(errs, key=errs.get)
@@ -137,6 +139,7 @@ def assert_matches_plain(got, model_dir, requests, dtype, what=""):
     own = row_errors({k: plain_logits(model_dir, requests, torch.bfloat16)[k[0]][k[1]]
                       for k in got}, ref)
     yard = float(np.sqrt(np.mean(np.square(list(own.values())))))
-    over = [k for k, e in errs.items() if e > 3 * yard]
-    assert errs[worst] < 6 * yard, (what, worst, errs[worst], yard)
+    bad = [k for k, e in errs.items() if e > max(6 * yard, 1.5 * own[k])]
+    over = [k for k, e in errs.items() if e > max(3 * yard, 1.5 * own[k])]
+    assert not bad, (what, bad[:5], [errs[k] for k in bad[:5]], yard)
     assert len(over) <= max(1, len(errs) // 50), (what, len(over), len(errs), yard, over[:5])
