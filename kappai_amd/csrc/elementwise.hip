@@ -63,17 +63,56 @@ extern "C" int kappai_embed_rows(const int* ids, const void* table, int table_is
 // * w, then resid += n (or resid = n), and the new resid again in the compute dtype for the next
 // sublayer to read.  a may come as `a_parts` float planes [parts][T][D] that are added in order
 // first (a product cut over its input dimension).  Everything in float32; a block a row, the row
-// kept in LDS between the sum of squares and the scaling.
+// kept in LDS between the sum of squares and the scaling.  `vec`: D is a multiple of eight and
+// every pointer of 32 bytes, so a thread takes eight values at a time and asks for the planes
+// four at a time (same sums in the same order).
 // ---------------------------------------------------------------------------------------
 template <typename TA, typename TO>
 __global__ __launch_bounds__(256) void output_norm_add_kernel(
     const TA* __restrict__ a, int a_parts, size_t a_plane, float scale_a, const TA* __restrict__ b,
     float scale_b, const float* __restrict__ w, float eps, float* __restrict__ resid, int add,
-    TO* __restrict__ rows, int D) {
-  extern __shared__ float ys[];
+    TO* __restrict__ rows, int D, int vec) {
+  extern __shared__ __attribute__((aligned(16))) float ys[];
   __shared__ float red[16];
   const size_t at = (size_t)blockIdx.x * D;
   float ss = 0.f;
+  if (vec) {
+    for (int e = 8 * threadIdx.x; e < D; e += 8 * 256) {
+      float v[8];
+      load8(a + at + e, v);
+#pragma unroll 4
+      for (int k = 1; k < a_parts; ++k) {
+        float u[8];
+        load8(a + k * a_plane + at + e, u);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] += u[i];
+      }
+      float bb[8];
+      if (b != nullptr) load8(b + at + e, bb);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        v[i] *= scale_a;
+        if (b != nullptr) v[i] = fmaf(scale_b, bb[i], v[i]);
+        ss = fmaf(v[i], v[i], ss);
+      }
+      store8(ys + e, v);
+    }
+    const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)D + eps);
+    for (int e = 8 * threadIdx.x; e < D; e += 8 * 256) {
+      float y[8], ww[8], r[8];
+      load8(ys + e, y);
+      load8(w + e, ww);
+      if (add) load8(resid + at + e, r);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        y[i] = y[i] * inv * ww[i];
+        if (add) y[i] += r[i];
+      }
+      store8(resid + at + e, y);
+      if (rows != nullptr) store8(rows + at + e, y);
+    }
+    return;
+  }
   for (int e = threadIdx.x; e < D; e += 256) {
     float v = to_f32(a[at + e]);
     for (int k = 1; k < a_parts; ++k) v += to_f32(a[k * a_plane + at + e]);
@@ -99,10 +138,12 @@ extern "C" int kappai_output_norm_add(const void* a, int a_is_bf16, int a_parts,
   if (D < 1 || D > 15 * 1024 || a_parts < 1 || (a_is_bf16 && a_parts != 1))
     return (int)hipErrorInvalidValue;
   const size_t lds = (size_t)D * sizeof(float), plane = (size_t)T * D;
+  const int vec = D % 8 == 0 && ((uintptr_t)a | (uintptr_t)b | (uintptr_t)w | (uintptr_t)resid |
+                                 (uintptr_t)rows) % 32 == 0;
 #define KAPPAI_OUT_NORM(TA, TO)                                                                  \
   hipLaunchKernelGGL((output_norm_add_kernel<TA, TO>), dim3(T), dim3(256), lds, stream,          \
                      (const TA*)a, a_parts, plane, scale_a, (const TA*)b, scale_b, w, eps, resid, \
-                     add, (TO*)rows, D)
+                     add, (TO*)rows, D, vec)
   if (a_is_bf16) {
     if (rows_is_bf16) KAPPAI_OUT_NORM(bf16_t, bf16_t); else KAPPAI_OUT_NORM(bf16_t, float);
   } else {

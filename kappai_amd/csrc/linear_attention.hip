@@ -1,4 +1,5 @@
-// Recurrences whose state is a matrix per head, S [d, dv] in float32 (a slot per request), with a
+// Recurrences whose state is a matrix per head, S [d, dv] in float32 (a slot per request; kept
+// column by column, [dv, d]), with a
 // decay per key channel:
 //   gated linear attention   S <- diag(a) S + k v^T                      o = S^T q
 //   gated delta rule         S <- diag(a) S; u = beta (v - S^T k); S <- S + k u^T;  o = S^T q
@@ -162,22 +163,245 @@ extern "C" int kappai_recurrence_prep(const void* q, int q_stride, const void* k
 }
 
 // ---------------------------------------------------------------------------------------
-// The recurrence itself.  A wave takes 64 / KS value channels of one (segment, head); lane
-// (c, s) keeps rows s * R .. s * R + R - 1 of column c in registers.  DELTA: the delta rule (needs
-// beta), else the plain gated sum.  Loads of the next token are asked for before the current one
-// is worked on.
+// The recurrence itself.  Lane (c, s) of a wave keeps R rows of column c of S in registers (eight;
+// sixteen for key sizes beyond 512), in groups of four: rows 4 (j KS + s) .. + 3 for j = 0 ..
+// R / 4 - 1, so that the KS lanes of a column read neighbouring 16-byte pieces of q, k and the
+// decay (no two on one LDS bank).  Few rows a lane, because a wave alone on its SIMD issues an
+// instruction only every ten cycles or so: the walk along the tokens is as fast as a wave's
+// instructions per token are few, and idle SIMDs are there to take more waves.  These lanes
+// are neighbours, and their partial dot products meet by data-parallel moves.  DELTA: the delta rule (needs beta), else the plain gated sum.
+// In memory a head's matrix lies column by column: state [slots, H, dv, d], so that a lane's rows
+// are consecutive and a wave's columns one stretch.
+//
+// Two kernels.  The block form: up to four waves share the q, k and decay rows of their head
+// (two when the grid would not fill the chip otherwise: what a CU's waves read from LDS per token
+// bounds the walk, so a long prompt's waves are spread over more CUs).
+// The tokens of a segment come in chunks of `tb`: while a chunk is worked on out of LDS, every
+// thread already holds its share of the next chunk's loads in registers, so the walk along the
+// tokens never waits for global memory.  The wave form reads each token from global memory one
+// ahead; it serves the shapes whose rows do not fit the block form's registers.
 // ---------------------------------------------------------------------------------------
-#define LA_R 16
+#define LA_MAX_WAVES 4
+#define LA_MAX_CHUNK 16
+
+// the r-th of a lane's rows
+template <int KS>
+__device__ __forceinline__ int la_row(int s, int r) { return 4 * ((r / 4) * KS + s) + r % 4; }
 
 template <int KS>
 __device__ __forceinline__ float ks_sum(float v) {
-#pragma unroll
-  for (int m = 1; m < KS; m <<= 1) v += __shfl_xor(v, m, WAVE);
+  if (KS >= 2) v += dpp_move<0xB1>(v);      // quad_perm [1, 0, 3, 2]
+  if (KS >= 4) v += dpp_move<0x4E>(v);      // quad_perm [2, 3, 0, 1]
+  if (KS >= 8) v += dpp_move<0x141>(v);     // the other quad of a half row (row_half_mirror)
+  if (KS >= 16) v += dpp_move<0x140>(v);    // the other half of a row (row_mirror)
+  if (KS >= 32) v += lane_xor16(v);
+  if (KS >= 64) v += lane_xor32(v);
   return v;
 }
 
-template <int KS, bool DELTA, typename TV>
-__global__ __launch_bounds__(WAVE) void matrix_state_scan_kernel(
+template <int KS, int R>
+__device__ __forceinline__ void la_load_rows(const float* __restrict__ st, int s, int d,
+                                             bool carry, float (&S)[R]) {
+#pragma unroll
+  for (int r = 0; r < R; ++r) S[r] = 0.f;
+  if (!carry) return;
+  if (d % 4 == 0) {
+#pragma unroll
+    for (int r4 = 0; r4 < R; r4 += 4) {
+      const int row = la_row<KS>(s, r4);
+      if (row < d) {
+        const float4 x = *reinterpret_cast<const float4*>(st + row);
+        S[r4] = x.x; S[r4 + 1] = x.y; S[r4 + 2] = x.z; S[r4 + 3] = x.w;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (la_row<KS>(s, r) < d) S[r] = st[la_row<KS>(s, r)];
+  }
+}
+
+template <int KS, int R>
+__device__ __forceinline__ void la_store_rows(float* __restrict__ st, int s, int d,
+                                              const float (&S)[R]) {
+  if (d % 4 == 0) {
+#pragma unroll
+    for (int r4 = 0; r4 < R; r4 += 4) {
+      const int row = la_row<KS>(s, r4);
+      if (row < d)
+        *reinterpret_cast<float4*>(st + row) =
+            make_float4(S[r4], S[r4 + 1], S[r4 + 2], S[r4 + 3]);
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (la_row<KS>(s, r) < d) st[la_row<KS>(s, r)] = S[r];
+  }
+}
+
+// One token: S, the lane's rows of q, k and the decay, the column's v, the head's beta.  The dot
+// products are summed in four strands (rows r, r + 4, ...) that meet at the end: four short
+// chains of dependent operations instead of one long one.
+template <int KS, int R, bool DELTA>
+__device__ __forceinline__ float la_token(float (&S)[R], const float (&qc)[R],
+                                          const float (&kc)[R], const float (&ac)[R],
+                                          float vc, float bc) {
+  float o[4] = {0.f, 0.f, 0.f, 0.f};
+  if (DELTA) {
+    float dot[4] = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      S[r] *= ac[r];
+      dot[r % 4] = fmaf(S[r], kc[r], dot[r % 4]);
+    }
+    const float u = bc * (vc - ks_sum<KS>((dot[0] + dot[1]) + (dot[2] + dot[3])));
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      S[r] = fmaf(kc[r], u, S[r]);
+      o[r % 4] = fmaf(S[r], qc[r], o[r % 4]);
+    }
+  } else {
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      S[r] = fmaf(ac[r], S[r], kc[r] * vc);
+      o[r % 4] = fmaf(S[r], qc[r], o[r % 4]);
+    }
+  }
+  return ks_sum<KS>((o[0] + o[1]) + (o[2] + o[3]));
+}
+
+// LDS, per token of a chunk: q [dp], k [dp], a [dp] (dp = KS * R, zeros beyond d), v [NWC], beta,
+// padded to `rec` floats (a multiple of four).  d is a multiple of four and NWC a power of two
+// (1 << nwc_log2).  A thread's places in a chunk are fixed: LA_QS 16-byte pieces of each of q, k
+// and the decay (piece i = tid + j * threads: token i / (d / 4), floats 4 (i % (d / 4)) ..), and
+// up to LA_MAX_CHUNK values of v.
+#define LA_QS 4
+template <int KS, int R, bool DELTA, typename TV>
+__global__ __launch_bounds__(LA_MAX_WAVES * WAVE) void matrix_state_scan_block_kernel(
+    const float* __restrict__ qf, const float* __restrict__ kf, const float* __restrict__ af,
+    const float* __restrict__ bf, const TV* __restrict__ v, int v_stride,
+    float* __restrict__ state, const int* __restrict__ seg_start,
+    const int* __restrict__ seg_pos0, const int* __restrict__ seg_slot, int H, int Hk, int d,
+    int dv, int tb, int rec, int nwc_log2, float* __restrict__ out) {
+  extern __shared__ float sh_scan[];
+  constexpr int COLS = WAVE / KS;
+  constexpr int DP = KS * R;
+  const int nthr = blockDim.x, tid = threadIdx.x, lane = tid % WAVE, wave = tid / WAVE;
+  const int NWC = 1 << nwc_log2;
+  const int seg = blockIdx.z, h = blockIdx.y, c0 = blockIdx.x * NWC;
+  const int s = lane % KS, cl = wave * COLS + lane / KS, c = c0 + cl;
+  const bool col_ok = c < dv;
+  const int cc = col_ok ? c : dv - 1;
+  const int hk = h / (H / Hk);
+  const int first = seg_start[seg], last = seg_start[seg + 1];
+  float* st = state + (((size_t)seg_slot[seg] * H + h) * dv + cc) * d;
+  float S[R];
+  la_load_rows<KS, R>(st, s, d, seg_pos0[seg] > 0, S);
+
+  // the thread's places
+  const int g4 = d / 4;
+  int p_tok[LA_QS], p_qk[LA_QS], p_a[LA_QS], p_lds[LA_QS];
+#pragma unroll
+  for (int j = 0; j < LA_QS; ++j) {
+    const int i = tid + j * nthr, tt = i / g4, g = i - tt * g4;
+    p_tok[j] = tt;
+    p_qk[j] = (tt * Hk + hk) * d + 4 * g;
+    p_a[j] = (tt * H + h) * d + 4 * g;
+    p_lds[j] = tt * rec + 4 * g;
+  }
+  const int v_slots = (tb * NWC + nthr - 1) / nthr;
+  const int v_col = min(c0 + (tid & (NWC - 1)), dv - 1);
+  float4 sq[LA_QS], sk[LA_QS], sa[LA_QS];
+  float sv[LA_MAX_CHUNK], sb = 0.f;
+  // the thread's share of the chunk that starts at token t0 (n tokens), into registers ...
+  auto fetch = [&](int t0, int n) {
+    const float* qb = qf + (size_t)t0 * Hk * d;
+    const float* kb = kf + (size_t)t0 * Hk * d;
+    const float* ab = af + (size_t)t0 * H * d;
+#pragma unroll
+    for (int j = 0; j < LA_QS; ++j)
+      if (p_tok[j] < n) {
+        sq[j] = *reinterpret_cast<const float4*>(qb + p_qk[j]);
+        sk[j] = *reinterpret_cast<const float4*>(kb + p_qk[j]);
+        sa[j] = *reinterpret_cast<const float4*>(ab + p_a[j]);
+      }
+#pragma unroll
+    for (int j = 0; j < LA_MAX_CHUNK; ++j)
+      if (j < v_slots) {
+        const int tt = (tid + j * nthr) >> nwc_log2;
+        if (tt < n) sv[j] = to_f32(v[(size_t)(t0 + tt) * v_stride + (size_t)h * dv + v_col]);
+      }
+    if (DELTA && tid < n) sb = bf[(size_t)(t0 + tid) * H + h];
+  };
+  // ... and from the registers to LDS
+  auto put = [&](int n) {
+#pragma unroll
+    for (int j = 0; j < LA_QS; ++j)
+      if (p_tok[j] < n) {
+        *reinterpret_cast<float4*>(sh_scan + p_lds[j]) = sq[j];
+        *reinterpret_cast<float4*>(sh_scan + p_lds[j] + DP) = sk[j];
+        *reinterpret_cast<float4*>(sh_scan + p_lds[j] + 2 * DP) = sa[j];
+      }
+#pragma unroll
+    for (int j = 0; j < LA_MAX_CHUNK; ++j)
+      if (j < v_slots) {
+        const int i = tid + j * nthr, tt = i >> nwc_log2;
+        if (tt < n) sh_scan[tt * rec + 3 * DP + (i & (NWC - 1))] = sv[j];
+      }
+    if (DELTA && tid < n) sh_scan[tid * rec + 3 * DP + NWC] = sb;
+  };
+  // a token's values for this lane out of LDS
+  auto read = [&](int tt, float (&q_)[R], float (&k_)[R], float (&a_)[R], float& v_,
+                  float& b_) {
+    const float* base = sh_scan + tt * rec;
+#pragma unroll
+    for (int r4 = 0; r4 < R; r4 += 4) {
+      const int row = la_row<KS>(s, r4);
+      const float4 x = *reinterpret_cast<const float4*>(base + row);
+      const float4 y = *reinterpret_cast<const float4*>(base + DP + row);
+      const float4 z = *reinterpret_cast<const float4*>(base + 2 * DP + row);
+      q_[r4] = x.x; q_[r4 + 1] = x.y; q_[r4 + 2] = x.z; q_[r4 + 3] = x.w;
+      k_[r4] = y.x; k_[r4 + 1] = y.y; k_[r4 + 2] = y.z; k_[r4 + 3] = y.w;
+      a_[r4] = z.x; a_[r4 + 1] = z.y; a_[r4 + 2] = z.z; a_[r4 + 3] = z.w;
+    }
+    v_ = base[3 * DP + cl];
+    b_ = base[3 * DP + NWC];
+  };
+  int n = min(tb, last - first);
+  if (n > 0) fetch(first, n);
+  for (int i = tid; i < tb * rec; i += nthr) sh_scan[i] = 0.f;     // (the zeros beyond d stay)
+  __syncthreads();
+  if (n > 0) put(n);
+  __syncthreads();
+  float* orow = out + (size_t)h * dv + c;
+  const size_t ostep = (size_t)H * dv;
+  const bool writes = s == 0 && col_ok;
+  for (int t0 = first; t0 < last; t0 += tb) {
+    n = min(tb, last - t0);
+    const int nn = min(tb, last - t0 - tb);
+    if (nn > 0) fetch(t0 + tb, nn);
+    // two sets of registers take turns: one is read for the next token while the other is used
+    float q0[R], k0[R], a0[R], v0, b0, q1[R], k1[R], a1[R], v1, b1;
+    read(0, q0, k0, a0, v0, b0);
+    for (int tt = 0; tt < n; tt += 2) {
+      if (tt + 1 < n) read(tt + 1, q1, k1, a1, v1, b1);
+      const float o0 = la_token<KS, R, DELTA>(S, q0, k0, a0, v0, b0);
+      if (writes) orow[(size_t)(t0 + tt) * ostep] = o0;
+      if (tt + 1 < n) {
+        if (tt + 2 < n) read(tt + 2, q0, k0, a0, v0, b0);
+        const float o1 = la_token<KS, R, DELTA>(S, q1, k1, a1, v1, b1);
+        if (writes) orow[(size_t)(t0 + tt + 1) * ostep] = o1;
+      }
+    }
+    __syncthreads();
+    if (nn > 0) put(nn);
+    __syncthreads();
+  }
+  if (col_ok) la_store_rows<KS, R>(st, s, d, S);
+}
+
+template <int KS, int R, bool DELTA, typename TV>
+__global__ __launch_bounds__(WAVE) void matrix_state_scan_wave_kernel(
     const float* __restrict__ qf, const float* __restrict__ kf, const float* __restrict__ af,
     const float* __restrict__ bf, const TV* __restrict__ v, int v_stride,
     float* __restrict__ state, const int* __restrict__ seg_start,
@@ -189,109 +413,124 @@ __global__ __launch_bounds__(WAVE) void matrix_state_scan_kernel(
   const bool col_ok = c < dv;
   const int cc = col_ok ? c : dv - 1;
   const int hk = h / (H / Hk);
-  const int r0 = s * LA_R;
   const int first = seg_start[seg], last = seg_start[seg + 1];
-  float* st = state + (((size_t)seg_slot[seg] * H + h) * d) * dv + cc;
-  float S[LA_R];
-  const bool carry = seg_pos0[seg] > 0;
-#pragma unroll
-  for (int r = 0; r < LA_R; ++r)
-    S[r] = (carry && r0 + r < d) ? st[(size_t)(r0 + r) * dv] : 0.f;
+  float* st = state + (((size_t)seg_slot[seg] * H + h) * dv + cc) * d;
+  float S[R];
+  la_load_rows<KS, R>(st, s, d, seg_pos0[seg] > 0, S);
 
-  float qn[LA_R], kn[LA_R], an[LA_R], vn = 0.f, bn = 0.f;
+  float qn[R], kn[R], an[R], vn = 0.f, bn = 0.f;
   auto fetch = [&](int t) {
-    const float* qr = qf + ((size_t)t * Hk + hk) * d + r0;
-    const float* kr = kf + ((size_t)t * Hk + hk) * d + r0;
-    const float* ar = af + ((size_t)t * H + h) * d + r0;
+    const float* qr = qf + ((size_t)t * Hk + hk) * d;
+    const float* kr = kf + ((size_t)t * Hk + hk) * d;
+    const float* ar = af + ((size_t)t * H + h) * d;
 #pragma unroll
-    for (int r = 0; r < LA_R; ++r) {
-      const bool ok = r0 + r < d;
-      qn[r] = ok ? qr[r] : 0.f;
-      kn[r] = ok ? kr[r] : 0.f;
-      an[r] = ok ? ar[r] : 0.f;
+    for (int r = 0; r < R; ++r) {
+      const int row = la_row<KS>(s, r);
+      const bool ok = row < d;
+      qn[r] = ok ? qr[row] : 0.f;
+      kn[r] = ok ? kr[row] : 0.f;
+      an[r] = ok ? ar[row] : 0.f;
     }
     vn = to_f32(v[(size_t)t * v_stride + (size_t)h * dv + cc]);
     if (DELTA) bn = bf[(size_t)t * H + h];
   };
   if (first < last) fetch(first);
   for (int t = first; t < last; ++t) {
-    float qc[LA_R], kc[LA_R], ac[LA_R];
+    float qc[R], kc[R], ac[R];
 #pragma unroll
-    for (int r = 0; r < LA_R; ++r) { qc[r] = qn[r]; kc[r] = kn[r]; ac[r] = an[r]; }
+    for (int r = 0; r < R; ++r) { qc[r] = qn[r]; kc[r] = kn[r]; ac[r] = an[r]; }
     const float vc = vn, bc = bn;
     if (t + 1 < last) fetch(t + 1);
-    float o = 0.f;
-    if (DELTA) {
-      float dot = 0.f;
-#pragma unroll
-      for (int r = 0; r < LA_R; ++r) {
-        S[r] *= ac[r];
-        dot = fmaf(S[r], kc[r], dot);
-      }
-      dot = ks_sum<KS>(dot);
-      const float u = bc * (vc - dot);
-#pragma unroll
-      for (int r = 0; r < LA_R; ++r) {
-        S[r] = fmaf(kc[r], u, S[r]);
-        o = fmaf(S[r], qc[r], o);
-      }
-    } else {
-#pragma unroll
-      for (int r = 0; r < LA_R; ++r) {
-        S[r] = fmaf(ac[r], S[r], kc[r] * vc);
-        o = fmaf(S[r], qc[r], o);
-      }
-    }
-    o = ks_sum<KS>(o);
+    const float o = la_token<KS, R, DELTA>(S, qc, kc, ac, vc, bc);
     if (s == 0 && col_ok) out[(size_t)t * H * dv + (size_t)h * dv + c] = o;
   }
-  if (col_ok) {
-#pragma unroll
-    for (int r = 0; r < LA_R; ++r)
-      if (r0 + r < d) st[(size_t)(r0 + r) * dv] = S[r];
-  }
+  if (col_ok) la_store_rows<KS, R>(st, s, d, S);
 }
 
-template <int KS, bool DELTA>
+// The block form's shape for a problem: waves a block (a power of two up to four, no more than
+// the columns ask for; halved while that leaves CUs without a block), tokens a chunk (0: the
+// shape does not fit and the wave form runs).
+struct LaBlockShape { int nw, tb, nwc_log2, rec; };
+#define LA_LDS_FLOATS 12288      // 48 KB
+static LaBlockShape la_block_shape(int ks, int r, int H, int S, int d, int dv) {
+  const int cols = WAVE / ks, col_waves = (dv + cols - 1) / cols;
+  int nw = 1;
+  while (nw * 2 <= LA_MAX_WAVES && nw < col_waves) nw *= 2;
+  while (nw > 2 && (long long)H * S * ((col_waves + nw - 1) / nw) < 256) nw /= 2;
+  int lg = 0;
+  while ((1 << lg) < nw * cols) ++lg;
+  const int rec = 3 * ks * r + ((nw * cols + 1 + 3) & ~3);
+  int tb = d % 4 ? 0 : LA_QS * nw * WAVE / (d / 4);
+  if (tb > LA_MAX_CHUNK) tb = LA_MAX_CHUNK;
+  if (tb > LA_LDS_FLOATS / rec) tb = LA_LDS_FLOATS / rec;
+  return LaBlockShape{nw, tb, lg, rec};
+}
+
+template <int KS, int R, bool DELTA, typename TV>
+static void scan_launch_typed(const float* qf, const float* kf, const float* af, const float* bf,
+                              const TV* v, int v_stride, float* state, const int* seg_start,
+                              const int* seg_pos0, const int* seg_slot, int S, int H, int Hk,
+                              int d, int dv, int form, float* out, hipStream_t stream) {
+  constexpr int COLS = WAVE / KS;
+  const LaBlockShape b = la_block_shape(KS, R, H, S, d, dv);
+  if (form == 1 || b.tb < 1) {
+    hipLaunchKernelGGL((matrix_state_scan_wave_kernel<KS, R, DELTA, TV>),
+                       dim3((dv + COLS - 1) / COLS, H, S), dim3(WAVE), 0, stream, qf, kf, af, bf,
+                       v, v_stride, state, seg_start, seg_pos0, seg_slot, H, Hk, d, dv, out);
+    return;
+  }
+  const int nwc = b.nw * COLS;
+  hipLaunchKernelGGL((matrix_state_scan_block_kernel<KS, R, DELTA, TV>),
+                     dim3((dv + nwc - 1) / nwc, H, S), dim3(b.nw * WAVE),
+                     (size_t)b.tb * b.rec * sizeof(float), stream, qf, kf, af, bf, v, v_stride,
+                     state, seg_start, seg_pos0, seg_slot, H, Hk, d, dv, b.tb, b.rec, b.nwc_log2,
+                     out);
+}
+
+template <int KS, int R, bool DELTA>
 static void scan_launch(const float* qf, const float* kf, const float* af, const float* bf,
                         const void* v, int v_stride, int v_is_bf16, float* state,
                         const int* seg_start, const int* seg_pos0, const int* seg_slot, int S,
-                        int H, int Hk, int d, int dv, float* out, hipStream_t stream) {
-  constexpr int COLS = WAVE / KS;
-  dim3 grid((dv + COLS - 1) / COLS, H, S);
+                        int H, int Hk, int d, int dv, int form, float* out, hipStream_t stream) {
   if (v_is_bf16)
-    hipLaunchKernelGGL((matrix_state_scan_kernel<KS, DELTA, bf16_t>), grid, dim3(WAVE), 0, stream,
-                       qf, kf, af, bf, (const bf16_t*)v, v_stride, state, seg_start, seg_pos0,
-                       seg_slot, H, Hk, d, dv, out);
+    scan_launch_typed<KS, R, DELTA, bf16_t>(qf, kf, af, bf, (const bf16_t*)v, v_stride, state,
+                                         seg_start, seg_pos0, seg_slot, S, H, Hk, d, dv, form,
+                                         out, stream);
   else
-    hipLaunchKernelGGL((matrix_state_scan_kernel<KS, DELTA, float>), grid, dim3(WAVE), 0, stream,
-                       qf, kf, af, bf, (const float*)v, v_stride, state, seg_start, seg_pos0,
-                       seg_slot, H, Hk, d, dv, out);
+    scan_launch_typed<KS, R, DELTA, float>(qf, kf, af, bf, (const float*)v, v_stride, state,
+                                        seg_start, seg_pos0, seg_slot, S, H, Hk, d, dv, form, out,
+                                        stream);
 }
 
+// form: 0 = the block form where it fits, 1 = the wave form, 2 = the block form or an error.
 extern "C" int kappai_matrix_state_scan(const float* qf, const float* kf, const float* af,
                                         const float* bf, const void* v, int v_stride,
                                         int v_is_bf16, float* state, const int* seg_start,
                                         const int* seg_pos0, const int* seg_slot, int T, int S,
-                                        int H, int Hk, int d, int dv, int delta, float* out,
-                                        hipStream_t stream) {
+                                        int H, int Hk, int d, int dv, int delta, int form,
+                                        float* out, hipStream_t stream) {
   if (T <= 0 || S <= 0) return 0;
-  if (H < 1 || Hk < 1 || H % Hk || H > 65535 || S > 65535 || d < 1 || d > 64 * LA_R || dv < 1)
+  if (H < 1 || Hk < 1 || H % Hk || H > 65535 || S > 65535 || d < 1 || d > 64 * 16 || dv < 1 ||
+      form < 0 || form > 2)
     return (int)hipErrorInvalidValue;
   if (delta && bf == nullptr) return (int)hipErrorInvalidValue;
+  // eight rows a lane; sixteen for the key sizes that 64 lanes of eight do not hold
+  const int r = d <= 64 * 8 ? 8 : 16;
   int ks = 1;
-  while (ks * LA_R < d) ks *= 2;
-#define LA_CASE(KS_)                                                                            \
-  case KS_:                                                                                     \
+  while (ks * r < d) ks *= 2;
+  if (form == 2 && la_block_shape(ks, r, H, S, d, dv).tb < 1) return (int)hipErrorInvalidValue;
+#define LA_CASE(KS_, R_)                                                                          \
+  case KS_ * 100 + R_:                                                                                    \
     if (delta)                                                                                  \
-      scan_launch<KS_, true>(qf, kf, af, bf, v, v_stride, v_is_bf16, state, seg_start, seg_pos0, \
-                             seg_slot, S, H, Hk, d, dv, out, stream);                           \
+      scan_launch<KS_, R_, true>(qf, kf, af, bf, v, v_stride, v_is_bf16, state, seg_start, seg_pos0, \
+                             seg_slot, S, H, Hk, d, dv, form, out, stream);                     \
     else                                                                                        \
-      scan_launch<KS_, false>(qf, kf, af, bf, v, v_stride, v_is_bf16, state, seg_start,         \
-                              seg_pos0, seg_slot, S, H, Hk, d, dv, out, stream);                \
+      scan_launch<KS_, R_, false>(qf, kf, af, bf, v, v_stride, v_is_bf16, state, seg_start,         \
+                              seg_pos0, seg_slot, S, H, Hk, d, dv, form, out, stream);          \
     break;
-  switch (ks) {
-    LA_CASE(1) LA_CASE(2) LA_CASE(4) LA_CASE(8) LA_CASE(16) LA_CASE(32) LA_CASE(64)
+  switch (ks * 100 + r) {
+    LA_CASE(1, 8) LA_CASE(2, 8) LA_CASE(4, 8) LA_CASE(8, 8) LA_CASE(16, 8) LA_CASE(32, 8)
+    LA_CASE(64, 8) LA_CASE(64, 16)
     default: return (int)hipErrorInvalidValue;
   }
 #undef LA_CASE

@@ -1801,15 +1801,18 @@ def conv_silu(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, row_pos:
     return out
 
 
+SCAN_FORMS = {"auto": 0, "wave": 1, "block": 2}
+
+
 def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor,
                             n_heads: int, n_qk_heads: int, dim: int, vdim: int,
                             rate: torch.Tensor, z_bias: Optional[torch.Tensor], z_sign: float,
                             q_scale: float, state: torch.Tensor, seg_start: torch.Tensor,
                             seg_pos0: torch.Tensor, seg_slot: torch.Tensor,
                             beta: Optional[torch.Tensor] = None, unit_qk: bool = False,
-                            unit_eps: float = 1e-6) -> torch.Tensor:
-    """A state ``S`` [dim, vdim] per head, float32, in ``state`` [slots, H, dim, vdim] (a segment
-    that starts at position 0 starts from zero).  Per token, with the decay per key channel
+                            unit_eps: float = 1e-6, form: str = "auto") -> torch.Tensor:
+    """A state ``S`` [dim, vdim] per head, float32, kept column by column in ``state``
+    [slots, H, vdim, dim] (a segment that starts at position 0 starts from zero).  Per token, with the decay per key channel
     ``a = exp(-rate[h] * softplus(z_sign * (z + z_bias)))``:
     without ``beta``   ``S <- diag(a) S + k v^T``, ``o = S^T q``;
     with ``beta``      ``S <- diag(a) S``, ``u = sigmoid(beta) (v - S^T k)``, ``S <- S + k u^T``,
@@ -1817,8 +1820,12 @@ def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z
     ``q``, ``k`` [T, Hk dim] (head h reads q/k head ``h // (H / Hk)``; ``unit_qk``: each head's
     vector divided by ``sqrt(sum x^2 + unit_eps)`` first), q times ``q_scale``; ``v`` [T, H vdim];
     ``z`` [T, H dim]; ``beta`` [T, H]; all views with a row stride.  Everything between the
-    projections and the result is float32.  Returns ``o`` [T, H vdim] float32."""
+    projections and the result is float32.  Returns ``o`` [T, H vdim] float32.
+
+    ``form`` = "wave" | "block" forces one of the two kernels (for tests): a wave that reads each
+    token from global memory, or a block of waves that takes the tokens in chunks through LDS."""
     H, Hk, d, dv = n_heads, n_qk_heads, dim, vdim
+    _need(form in SCAN_FORMS, lambda: f"matrix_state_recurrence: form {form!r}")
     T = q.shape[0]
     for name, t, cols in (("q", q, Hk * d), ("k", k, Hk * d), ("v", v, H * dv), ("z", z, H * d)):
         _gpu(name, t, q.dtype, contiguous=False)
@@ -1835,8 +1842,8 @@ def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z
         _gpu("z_bias", z_bias, F32)
         _need(z_bias.shape == (H * d,), "matrix_state_recurrence: z_bias must be [H dim]")
     _gpu("state", state, F32)
-    _need(tuple(state.shape[1:]) == (H, d, dv),
-          lambda: f"matrix_state_recurrence: state {tuple(state.shape)} for {H} x {d} x {dv}")
+    _need(tuple(state.shape[1:]) == (H, dv, d),
+          lambda: f"matrix_state_recurrence: state {tuple(state.shape)} for {H} x {dv} x {d}")
     for name, t in (("seg_start", seg_start), ("seg_pos0", seg_pos0), ("seg_slot", seg_slot)):
         _gpu(name, t, I32)
     S = seg_slot.shape[0]
@@ -1857,7 +1864,8 @@ def matrix_state_recurrence(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z
         _ptr(qf), _ptr(kf), _ptr(af), _ptr(bf), _ptr(v), _c_int(v.stride(0)),
         _c_int(_is_bf16(v.dtype)), _ptr(state), _ptr(seg_start), _ptr(seg_pos0), _ptr(seg_slot),
         _c_int(T), _c_int(S), _c_int(H), _c_int(Hk), _c_int(d), _c_int(dv),
-        _c_int(1 if beta is not None else 0), _ptr(out), _stream()), "matrix_state_scan")
+        _c_int(1 if beta is not None else 0), _c_int(SCAN_FORMS[form]), _ptr(out), _stream()),
+        "matrix_state_scan")
     return out
 
 

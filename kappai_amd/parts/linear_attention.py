@@ -63,7 +63,7 @@ class GatedLinearAttention(Mixer):
         self.decay_bias = self.norm_w = self.rate = None
 
     def cache_spec(self):
-        return FixedState((self.H, self.d, self.dv), "float32")
+        return FixedState((self.H, self.dv, self.d), "float32")
 
     def tensor_specs(self) -> List[TensorSpec]:
         return (self.inputs.tensor_specs() + self.decay.tensor_specs() + self.out.tensor_specs()
@@ -138,7 +138,7 @@ class GatedDeltaRule(Mixer):
         self.conv_taps = self.rate = self.dt_bias = self.norm_w = None
 
     def cache_spec(self):
-        state = FixedState((self.H, self.d, self.dv), "float32")
+        state = FixedState((self.H, self.dv, self.d), "float32")
         if self.taps == 1:
             return state
         return CacheBundle((("state", state),

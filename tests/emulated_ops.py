@@ -508,7 +508,7 @@ def conv_silu(x, taps, state, row_pos, row_seg, seg_start, seg_pos0, seg_slot):
 
 def matrix_state_recurrence(q, k, v, z, n_heads, n_qk_heads, dim, vdim, rate, z_bias, z_sign,
                             q_scale, state, seg_start, seg_pos0, seg_slot, beta=None,
-                            unit_qk=False, unit_eps=1e-6):
+                            unit_qk=False, unit_eps=1e-6, form="auto"):
     H, Hk, d, dv = n_heads, n_qk_heads, dim, vdim
     T = q.shape[0]
     qf = q[:, :Hk * d].to(F32).reshape(T, Hk, d)
@@ -527,7 +527,8 @@ def matrix_state_recurrence(q, k, v, z, n_heads, n_qk_heads, dim, vdim, rate, z_
     out = torch.empty((T, H, dv), dtype=F32)
     for s in range(seg_slot.shape[0]):
         t0, t1, slot = int(seg_start[s]), int(seg_start[s + 1]), int(seg_slot[s])
-        S = torch.zeros((H, d, dv)) if int(seg_pos0[s]) == 0 else state[slot].clone()
+        S = (torch.zeros((H, d, dv)) if int(seg_pos0[s]) == 0
+             else state[slot].transpose(1, 2).clone())
         for t in range(t0, t1):
             S = a[t][:, :, None] * S
             if b is not None:
@@ -536,7 +537,7 @@ def matrix_state_recurrence(q, k, v, z, n_heads, n_qk_heads, dim, vdim, rate, z_
                 u = vf[t]
             S = S + kf[t][:, :, None] * u[:, None, :]
             out[t] = torch.einsum("hdv,hd->hv", S, qf[t])
-        state[slot] = S
+        state[slot] = S.transpose(1, 2)
     return out.reshape(T, H * dv)
 
 

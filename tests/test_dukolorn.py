@@ -125,13 +125,13 @@ def test_what_the_layers_ask_of_the_cache_manager():
     specs = model.cache_specs()
     assert isinstance(specs[0], CacheBundle)
     assert specs[0].member("left") == PagedKV(2, 32, None)         # heads of 16 / 24 in one size
-    assert specs[0].member("right") == FixedState((3, 8, 16), "float32")
+    assert specs[0].member("right") == FixedState((3, 16, 8), "float32")
     assert specs[1] == PagedKV(1, 32, 21)                           # latent 20 + 8 rotated places
-    assert specs[2].member("state") == FixedState((4, 8, 16), "float32")
+    assert specs[2].member("state") == FixedState((4, 16, 8), "float32")
     assert specs[2].member("conv") == FixedState((2, 2 * 16 + 64), "float32")
     # one tap: the convolution keeps no history and the layer asks for its state alone
     v = build_model(config_from_dict(copy.deepcopy(TINY["V"][0])), "float32").cache_specs()
-    assert v[0] == FixedState((1, 24, 8), "float32")
+    assert v[0] == FixedState((1, 8, 24), "float32")
     cm = CacheManager(specs, 16, 8, 2)
     cm.allocate_storage(torch.float32, "cpu")
     assert len(cm.paged_groups) == 2 and cm.paged_groups[1].spec.window == 21
@@ -139,7 +139,7 @@ def test_what_the_layers_ask_of_the_cache_manager():
     cm.extend(rc, 40)
     cm.commit(rc, 40)
     assert rc.blocks[1][0] == -1 and rc.blocks[0][0] >= 0    # the window gave its first page back
-    assert cm.view(0).part("right").state.shape == (3, 3, 8, 16)
+    assert cm.view(0).part("right").state.shape == (3, 3, 16, 8)
     cm.close(rc)
     cm.check()
 
