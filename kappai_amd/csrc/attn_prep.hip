@@ -223,11 +223,69 @@ __global__ __launch_bounds__(256) void headwise_linear_kernel(
   }
 }
 
+// The same on the matrix cores, for bfloat16 with n_in, the strides and the pointers multiples of
+// eight values.  A wave takes 16 rows x 64 outputs of one head: per step of 32 along i a lane
+// loads eight values of its row of x (row lane % 16, values 8 (lane / 16) ..) and of four rows of
+// W the same way, and four products W-tile x x-tile^T add up; a lane ends with outputs
+// 16 j + 4 (lane / 16) .. + 3 of row lane % 16.  Four waves a block (64 rows); one when there are
+// no more than 16 rows.
+typedef __attribute__((ext_vector_type(8))) __bf16 hw_bf16x8_t;
+typedef __attribute__((ext_vector_type(4))) float hw_f32x4_t;
+
+__global__ __launch_bounds__(256) void headwise_linear_mfma_kernel(
+    const bf16_t* __restrict__ x, int x_row, int x_head, const bf16_t* __restrict__ w, int n_out,
+    int n_in, bf16_t* __restrict__ y, int y_row, int y_head, int rows) {
+  const int h = blockIdx.z, lane = threadIdx.x % WAVE, wave = threadIdx.x / WAVE;
+  const int m0 = (blockIdx.x * (blockDim.x / WAVE) + wave) * 16, n0 = blockIdx.y * 64;
+  if (m0 >= rows) return;
+  const int lr = lane % 16, kq = lane / 16;
+  const int m = min(m0 + lr, rows - 1);
+  const bf16_t* xr = x + (size_t)m * x_row + (size_t)h * x_head + 8 * kq;
+  const bf16_t* wr[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    wr[j] = w + ((size_t)h * n_out + min(n0 + 16 * j + lr, n_out - 1)) * n_in + 8 * kq;
+  hw_f32x4_t acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc[j] = (hw_f32x4_t){0.f, 0.f, 0.f, 0.f};
+  const uint4 zero = make_uint4(0u, 0u, 0u, 0u);
+  for (int k0 = 0; k0 < n_in; k0 += 32) {
+    const bool ok = k0 + 8 * kq < n_in;         // (n_in is a multiple of eight: all or nothing)
+    const uint4 xv = ok ? *reinterpret_cast<const uint4*>(xr + k0) : zero;
+    uint4 wv[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) wv[j] = ok ? *reinterpret_cast<const uint4*>(wr[j] + k0) : zero;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(hw_bf16x8_t, wv[j]),
+                                                       __builtin_bit_cast(hw_bf16x8_t, xv), acc[j],
+                                                       0, 0, 0);
+  }
+  if (m0 + lr >= rows) return;
+  bf16_t* yr = y + (size_t)(m0 + lr) * y_row + (size_t)h * y_head;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+      const int n = n0 + 16 * j + 4 * kq + v;
+      if (n < n_out) yr[n] = f32_to_bf16(acc[j][v]);
+    }
+}
+
 extern "C" int kappai_headwise_linear(const void* x, int x_row, int x_head, const void* w, int H,
                                       int n_out, int n_in, void* y, int y_row, int y_head,
                                       int rows, int is_bf16, hipStream_t stream) {
   if (rows <= 0) return 0;
   if (H < 1 || H > 65535 || n_out < 1 || n_in < 1) return (int)hipErrorInvalidValue;
+  if (is_bf16 && n_in % 8 == 0 && x_row % 8 == 0 && x_head % 8 == 0 &&
+      ((uintptr_t)x | (uintptr_t)w) % 16 == 0 && (n_out + 63) / 64 <= 65535) {
+    const int waves = rows <= 16 ? 1 : 4;
+    hipLaunchKernelGGL(headwise_linear_mfma_kernel,
+                       dim3((rows + 16 * waves - 1) / (16 * waves), (n_out + 63) / 64, H),
+                       dim3(waves * WAVE), 0, stream, (const bf16_t*)x, x_row, x_head,
+                       (const bf16_t*)w, n_out, n_in, (bf16_t*)y, y_row, y_head, rows);
+    KAPPAI_RETURN_LAUNCH_STATUS();
+  }
   dim3 grid((rows + HW_BM - 1) / HW_BM, (n_out + HW_BN - 1) / HW_BN, H);
   if (grid.y > 65535) return (int)hipErrorInvalidValue;
   if (is_bf16)

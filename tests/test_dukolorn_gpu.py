@@ -182,18 +182,25 @@ def test_matrix_state_recurrence_against_the_stand_in(H, Hk, d, dv, delta, form)
         assert rel(torch.cat(got[i]), want[i].double()) < 2e-5, i
 
 
-@pytest.mark.parametrize("H,n_in,n_out,T", [(3, 16, 20, 37), (1, 40, 8, 1), (4, 8, 100, 70),
-                                            (2, 33, 65, 5)])
+@pytest.mark.parametrize("H,n_in,n_out,T,pad", [(3, 16, 20, 37, 4), (1, 40, 8, 1, 4),
+                                                (4, 8, 100, 70, 4), (2, 33, 65, 5, 4),
+                                                (3, 16, 20, 37, 8), (1, 40, 8, 1, 0),
+                                                (4, 72, 100, 70, 16), (2, 192, 130, 16, 64),
+                                                (5, 24, 64, 17, 8), (2, 128, 192, 200, 0)])
 @pytest.mark.parametrize("dtype", [F32, BF16])
-def test_a_matrix_per_head(H, n_in, n_out, T, dtype):
+def test_a_matrix_per_head(H, n_in, n_out, T, pad, dtype):
+    """Heads that stand ``n_in + pad`` apart in rows of a few values more; in bfloat16 the paddings
+    that keep every head at a multiple of eight values run on the matrix cores, the others and
+    float32 on the plain kernel."""
     from kappai_amd.kernels import ops
-    x = torch.randn(T, H * (n_in + 4) + 3, generator=gen(9)).to(BF16)
+    step = n_in + pad
+    x = torch.randn(T, H * step + 8, generator=gen(9)).to(BF16)
     w = (torch.randn(H, n_out, n_in, generator=gen(10)) * 0.3).to(BF16)
     out = torch.zeros(T, H * (n_out + 2), dtype=dtype, device=DEV)
-    ops.headwise_linear(x.to(dtype).to(DEV), n_in + 4, w.to(dtype).to(DEV), out=out,
+    ops.headwise_linear(x.to(dtype).to(DEV), step, w.to(dtype).to(DEV), out=out,
                         out_head_stride=n_out + 2)
     for h in range(H):
-        want = x[:, h * (n_in + 4):h * (n_in + 4) + n_in].double() @ w[h].double().T
+        want = x[:, h * step:h * step + n_in].double() @ w[h].double().T
         got = out[:, h * (n_out + 2):h * (n_out + 2) + n_out]
         assert rel(got.float(), want) < (1e-5 if dtype == F32 else 1e-2)
         assert float(out[:, h * (n_out + 2) + n_out:(h + 1) * (n_out + 2)].abs().max()) == 0.0
