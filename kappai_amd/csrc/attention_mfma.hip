@@ -139,8 +139,12 @@ __device__ __forceinline__ u32x4_t load_k8(const bf16_t* __restrict__ k_pool,
 // longest chain of dependent work fourfold; their partial results meet in LDS
 #define P_NW (HEAD_DIM <= 128 ? 4 : 1)
 
-// MODS: the scores pass kappai_modified_score (a cap, a bias by distance) between the scaled
-// product and the softmax, and a sink may join the denominator (score_mods.h).
+// MODS: the scores pass a cap and a bias by distance between the scaled product and the softmax
+// (score_mods.h).  The head's row of the bias table lies in LDS (tables of up to P_BIAS_MAX
+// columns; longer ones are read where they are), and a key tile that is further from every query
+// of the block than the table reaches takes the table's last column without looking.  A sink may
+// join the denominator with or without MODS.
+#define P_BIAS_MAX 2048
 template <bool MODS>
 __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pool,
@@ -182,6 +186,16 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
   float m_run = -INFINITY, l_run = 0.f;
   // (with MODS the scores are scaled, worked on and brought to units of log 2 one by one)
   const float sc = MODS ? 1.0f : scale * LOG2E;
+  __shared__ float sh_bias[MODS ? P_BIAS_MAX : 1];
+  const bool has_bias = MODS && mods.dist_bias != nullptr;
+  const bool bias_in_lds = has_bias && mods.dist_cols <= P_BIAS_MAX;
+  const float* bias_row = has_bias ? mods.dist_bias + (size_t)h * mods.dist_cols : nullptr;
+  const float far_bias = has_bias ? bias_row[mods.dist_cols - 1] : 0.f;
+  if (MODS) {
+    if (bias_in_lds)
+      for (int i = threadIdx.x; i < mods.dist_cols; i += P_NW * WAVE) sh_bias[i] = bias_row[i];
+    __syncthreads();
+  }
 
   // A tile of 32 keys is "whole" when every row of the q tile sees all of its keys: then nothing
   // is masked, and addresses are a base that is the same for all lanes of a 16-key group (its
@@ -252,10 +266,22 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
       s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_frag(kfr[buf][ks]), qf[ks], s, 0, 0, 0);
     // lane holds, for query `col`, keys kb + 8*(v/4) + 4*hh + v%4
     if (MODS) {
+      const bool capped = mods.softcap > 0.f;
+      const bool far = has_bias && pos_first - (kb + 31) >= mods.dist_cols - 1;
 #pragma unroll
       for (int v = 0; v < 16; ++v) {
-        const int key = kb + 8 * (v / 4) + 4 * hh + v % 4;
-        s[v] = kappai_modified_score(mods, s[v] * scale, h, my_pos - key) * LOG2E;
+        float x = s[v] * scale;
+        if (capped) x = kappai_fast_cap(x, mods.softcap);
+        if (has_bias) {
+          if (far) {
+            x += far_bias;
+          } else {
+            const int key = kb + 8 * (v / 4) + 4 * hh + v % 4;
+            const int dist = max(0, min(my_pos - key, mods.dist_cols - 1));
+            x += bias_in_lds ? sh_bias[dist] : bias_row[dist];
+          }
+        }
+        s[v] = x * LOG2E;
       }
     }
     float mloc = -INFINITY;
@@ -347,7 +373,7 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
     l_run = sh_l[0][col];
 #pragma unroll
     for (int w = 1; w < P_NW; ++w) l_run += sh_l[w][col];
-    if (MODS && mods.sink != nullptr && M != -INFINITY)
+    if (mods.sink != nullptr && M != -INFINITY)
       l_run += fast_exp2(mods.sink[h] * LOG2E - M);
 #pragma unroll
     for (int mt = 0; mt < P_MT; ++mt)
@@ -360,7 +386,7 @@ __global__ __launch_bounds__(P_NW * WAVE) void attn_prefill_kernel(
       }
   }
   if (!row_ok) return;
-  if (MODS && P_NW == 1 && mods.sink != nullptr && m_run != -INFINITY)
+  if (P_NW == 1 && mods.sink != nullptr && m_run != -INFINITY)
     l_run += fast_exp2(mods.sink[h] * LOG2E - m_run);
   const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
   bf16_t* orow = out + (size_t)(r0 + col) * out_stride + (size_t)h * HEAD_DIM;
@@ -1050,9 +1076,14 @@ __device__ __forceinline__ void attn_decode_wave(
         for (int v = 0; v < 4; ++v) {
           const int key = kb + 8 * kg + 4 * tt + v;
           const bool ok = key >= lo && key <= hi;
-          if (MODS)
-            s[tt][v] = ok ? kappai_modified_score(*mods, s[tt][v] * scale, h, pos - key) * LOG2E
-                          : -INFINITY;
+          if (MODS) {
+            float x = s[tt][v] * scale;
+            if (mods->softcap > 0.f) x = kappai_fast_cap(x, mods->softcap);
+            if (mods->dist_bias != nullptr)
+              x += mods->dist_bias[(size_t)h * mods->dist_cols +
+                                   max(0, min(pos - key, mods->dist_cols - 1))];
+            s[tt][v] = ok ? x * LOG2E : -INFINITY;
+          }
           else
             s[tt][v] = ok ? s[tt][v] * sc : -INFINITY;
           mloc = fmaxf(mloc, s[tt][v]);
@@ -1263,7 +1294,7 @@ __global__ __launch_bounds__(D_BLOCK_MAX_WAVES * WAVE) void attn_decode_block_ke
       L += sh_l[w * 16 + c] * wgt;
       acc = fmaf(sh_o[((size_t)w * rep + c) * HEAD_DIM + e], wgt, acc);
     }
-    if (MODS && mods.sink != nullptr && M != -INFINITY)
+    if (mods.sink != nullptr && M != -INFINITY)
       L += fast_exp2(mods.sink[g * rep + c] * LOG2E - M);
     const float inv = L > 0.f ? 1.0f / L : 0.f;
     out[(size_t)t * out_stride + (size_t)(g * rep + c) * HEAD_DIM + e] = f32_to_bf16(acc * inv);
@@ -1395,7 +1426,7 @@ extern "C" int kappai_attn_decode_block_scored(const void* q, int q_stride, cons
     return (int)hipErrorInvalidValue;
   const int rep = H / G;
   const size_t lds = (size_t)n_waves * (rep * HEAD_DIM + 32) * sizeof(float);
-  if (kappai_mods_on(mods))
+  if (kappai_mods_change_scores(mods))
     hipLaunchKernelGGL(attn_decode_block_kernel<true>, dim3(T, G), dim3(n_waves * WAVE), lds,
                        stream, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool,
                        (const bf16_t*)vt_pool, (bf16_t*)out, out_stride, row_pos, row_seg,
@@ -1404,7 +1435,8 @@ extern "C" int kappai_attn_decode_block_scored(const void* q, int q_stride, cons
     hipLaunchKernelGGL(attn_decode_block_kernel<false>, dim3(T, G), dim3(n_waves * WAVE), lds,
                        stream, (const bf16_t*)q, q_stride, (const bf16_t*)k_pool,
                        (const bf16_t*)vt_pool, (bf16_t*)out, out_stride, row_pos, row_seg,
-                       block_tables, max_blocks, H, G, ps, window, scale, kappai_score_mods{0.f, nullptr, 0, nullptr});
+                       block_tables, max_blocks, H, G, ps, window, scale,
+                       kappai_score_mods{0.f, nullptr, 0, mods != nullptr ? mods->sink : nullptr});
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
@@ -1450,7 +1482,8 @@ extern "C" int kappai_attn_prefill_scored(const void* q, int q_stride, const voi
                                           int ps, int window, float scale, int variant,
                                           const kappai_score_mods* mods, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
-  if (kappai_mods_on(mods)) {
+  const float* sink = mods != nullptr ? mods->sink : nullptr;
+  if (kappai_mods_change_scores(mods)) {
     if (ps % 16 || G < 1 || H % G || H > 65535 || (q_stride % 8) || (out_stride % 4) ||
         variant == 2 || (mods->dist_bias != nullptr && mods->dist_cols < 1))
       return (int)hipErrorInvalidValue;
@@ -1464,10 +1497,12 @@ extern "C" int kappai_attn_prefill_scored(const void* q, int q_stride, const voi
     return (int)hipErrorInvalidValue;
   const int rep = H / G;
   const bool shared_ok = PG_OK && rep % 4 == 0;
-  if (variant == 2 && !shared_ok) return (int)hipErrorInvalidValue;
+  if (variant == 2 && (!shared_ok || sink != nullptr)) return (int)hipErrorInvalidValue;
   // sharing pays when there are blocks enough to fill the chip without splitting the keys of
   // a q tile over waves
-  const bool shared = variant == 2 || (variant == 0 && shared_ok && n_tiles * (H / 4) >= 256);
+  // (the kernel that shares key tiles knows no sink)
+  const bool shared = variant == 2 ||
+                      (variant == 0 && shared_ok && sink == nullptr && n_tiles * (H / 4) >= 256);
 #if PG_OK
   if (shared) {
     hipLaunchKernelGGL(attn_prefill_shared_kernel, dim3(n_tiles, H / 4), dim3(8 * WAVE), 0, stream,
@@ -1480,7 +1515,7 @@ extern "C" int kappai_attn_prefill_scored(const void* q, int q_stride, const voi
   hipLaunchKernelGGL(attn_prefill_kernel<false>, dim3(n_tiles, H), dim3(P_NW * WAVE), 0, stream,
                      (const bf16_t*)q, q_stride, (const bf16_t*)k_pool, (const bf16_t*)vt_pool,
                      (bf16_t*)out, out_stride, q_tiles, row_pos, block_tables, max_blocks, H, G,
-                     ps, window, scale, kappai_score_mods{0.f, nullptr, 0, nullptr});
+                     ps, window, scale, kappai_score_mods{0.f, nullptr, 0, sink});
   KAPPAI_RETURN_LAUNCH_STATUS();
 }
 
@@ -1501,9 +1536,10 @@ static int launch_decode(const void* q, int q_stride, const void* k_pool, const 
                          int keys_per_split, int n_splits, const QkFuse& qk, const int* row_ids,
                          hipStream_t stream, const kappai_score_mods* mods = nullptr) {
   if (T <= 0) return 0;
-  const bool scored = kappai_mods_on(mods);
+  const bool scored = kappai_mods_change_scores(mods);
   if (scored && qk.on) return (int)hipErrorInvalidValue;
-  const kappai_score_mods m = scored ? *mods : kappai_score_mods{0.f, nullptr, 0, nullptr};
+  const kappai_score_mods m =
+      scored ? *mods : kappai_score_mods{0.f, nullptr, 0, mods != nullptr ? mods->sink : nullptr};
   if (ps % 16 || G < 1 || H % G || H / G > 16 || G > 65535 || n_splits < 1 || n_splits > 65535 ||
       keys_per_split < D_KPW || keys_per_split % D_KPW || (q_stride % 8))
     return (int)hipErrorInvalidValue;

@@ -18,6 +18,18 @@ __host__ __device__ __forceinline__ bool kappai_mods_on(const kappai_score_mods*
   return m != nullptr && (m->softcap > 0.f || m->dist_bias != nullptr || m->sink != nullptr);
 }
 
+// (a cap or a bias: the scores themselves change; a sink alone leaves them as they are)
+__host__ __device__ __forceinline__ bool kappai_mods_change_scores(const kappai_score_mods* m) {
+  return m != nullptr && (m->softcap > 0.f || m->dist_bias != nullptr);
+}
+
+// cap * tanh(s / cap) for the kernels that work in bfloat16: tanh(x) = 1 - 2 / (1 + e^(2x)) by the
+// hardware's exponential and reciprocal (absolute error of a few 1e-7 of the cap).
+__device__ __forceinline__ float kappai_fast_cap(float s, float cap) {
+  const float e = __builtin_amdgcn_exp2f(s * (2.885390081777927f / cap));    // 2 log2(e) / cap
+  return cap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + e));
+}
+
 // `s` is the scaled dot product; the result is what the softmax sees (natural-logarithm units).
 __device__ __forceinline__ float kappai_modified_score(const kappai_score_mods& m, float s, int h,
                                                        int dist) {
