@@ -369,7 +369,8 @@ __global__ __launch_bounds__(LA_MAX_WAVES * WAVE) void matrix_state_scan_block_k
   };
   int n = min(tb, last - first);
   if (n > 0) fetch(first, n);
-  for (int i = tid; i < tb * rec; i += nthr) sh_scan[i] = 0.f;     // (the zeros beyond d stay)
+  // (the zeros beyond d stay; no more tokens' places than the segment will use)
+  for (int i = tid; i < min(tb, last - first) * rec; i += nthr) sh_scan[i] = 0.f;
   __syncthreads();
   if (n > 0) put(n);
   __syncthreads();
@@ -452,7 +453,7 @@ __global__ __launch_bounds__(WAVE) void matrix_state_scan_wave_kernel(
 // shape does not fit and the wave form runs).
 struct LaBlockShape { int nw, tb, nwc_log2, rec; };
 #define LA_LDS_FLOATS 12288      // 48 KB
-static LaBlockShape la_block_shape(int ks, int r, int H, int S, int d, int dv) {
+static LaBlockShape la_block_shape(int ks, int r, int H, int S, int T, int d, int dv) {
   const int cols = WAVE / ks, col_waves = (dv + cols - 1) / cols;
   int nw = 1;
   while (nw * 2 <= LA_MAX_WAVES && nw < col_waves) nw *= 2;
@@ -463,16 +464,17 @@ static LaBlockShape la_block_shape(int ks, int r, int H, int S, int d, int dv) {
   int tb = d % 4 ? 0 : LA_QS * nw * WAVE / (d / 4);
   if (tb > LA_MAX_CHUNK) tb = LA_MAX_CHUNK;
   if (tb > LA_LDS_FLOATS / rec) tb = LA_LDS_FLOATS / rec;
+  if (tb > T) tb = T;                 // (no segment is longer than the step)
   return LaBlockShape{nw, tb, lg, rec};
 }
 
 template <int KS, int R, bool DELTA, typename TV>
 static void scan_launch_typed(const float* qf, const float* kf, const float* af, const float* bf,
                               const TV* v, int v_stride, float* state, const int* seg_start,
-                              const int* seg_pos0, const int* seg_slot, int S, int H, int Hk,
-                              int d, int dv, int form, float* out, hipStream_t stream) {
+                              const int* seg_pos0, const int* seg_slot, int T, int S, int H,
+                              int Hk, int d, int dv, int form, float* out, hipStream_t stream) {
   constexpr int COLS = WAVE / KS;
-  const LaBlockShape b = la_block_shape(KS, R, H, S, d, dv);
+  const LaBlockShape b = la_block_shape(KS, R, H, S, T, d, dv);
   if (form == 1 || b.tb < 1) {
     hipLaunchKernelGGL((matrix_state_scan_wave_kernel<KS, R, DELTA, TV>),
                        dim3((dv + COLS - 1) / COLS, H, S), dim3(WAVE), 0, stream, qf, kf, af, bf,
@@ -490,16 +492,17 @@ static void scan_launch_typed(const float* qf, const float* kf, const float* af,
 template <int KS, int R, bool DELTA>
 static void scan_launch(const float* qf, const float* kf, const float* af, const float* bf,
                         const void* v, int v_stride, int v_is_bf16, float* state,
-                        const int* seg_start, const int* seg_pos0, const int* seg_slot, int S,
-                        int H, int Hk, int d, int dv, int form, float* out, hipStream_t stream) {
+                        const int* seg_start, const int* seg_pos0, const int* seg_slot, int T,
+                        int S, int H, int Hk, int d, int dv, int form, float* out,
+                        hipStream_t stream) {
   if (v_is_bf16)
     scan_launch_typed<KS, R, DELTA, bf16_t>(qf, kf, af, bf, (const bf16_t*)v, v_stride, state,
-                                         seg_start, seg_pos0, seg_slot, S, H, Hk, d, dv, form,
+                                         seg_start, seg_pos0, seg_slot, T, S, H, Hk, d, dv, form,
                                          out, stream);
   else
     scan_launch_typed<KS, R, DELTA, float>(qf, kf, af, bf, (const float*)v, v_stride, state,
-                                        seg_start, seg_pos0, seg_slot, S, H, Hk, d, dv, form, out,
-                                        stream);
+                                        seg_start, seg_pos0, seg_slot, T, S, H, Hk, d, dv, form,
+                                        out, stream);
 }
 
 // form: 0 = the block form where it fits, 1 = the wave form, 2 = the block form or an error.
@@ -518,15 +521,15 @@ extern "C" int kappai_matrix_state_scan(const float* qf, const float* kf, const 
   const int r = d <= 64 * 8 ? 8 : 16;
   int ks = 1;
   while (ks * r < d) ks *= 2;
-  if (form == 2 && la_block_shape(ks, r, H, S, d, dv).tb < 1) return (int)hipErrorInvalidValue;
+  if (form == 2 && la_block_shape(ks, r, H, S, T, d, dv).tb < 1) return (int)hipErrorInvalidValue;
 #define LA_CASE(KS_, R_)                                                                          \
   case KS_ * 100 + R_:                                                                                    \
     if (delta)                                                                                  \
       scan_launch<KS_, R_, true>(qf, kf, af, bf, v, v_stride, v_is_bf16, state, seg_start, seg_pos0, \
-                             seg_slot, S, H, Hk, d, dv, form, out, stream);                     \
+                             seg_slot, T, S, H, Hk, d, dv, form, out, stream);                     \
     else                                                                                        \
       scan_launch<KS_, R_, false>(qf, kf, af, bf, v, v_stride, v_is_bf16, state, seg_start,         \
-                              seg_pos0, seg_slot, S, H, Hk, d, dv, form, out, stream);          \
+                              seg_pos0, seg_slot, T, S, H, Hk, d, dv, form, out, stream);          \
     break;
   switch (ks * 100 + r) {
     LA_CASE(1, 8) LA_CASE(2, 8) LA_CASE(4, 8) LA_CASE(8, 8) LA_CASE(16, 8) LA_CASE(32, 8)
