@@ -46,7 +46,7 @@ def _python_flags() -> List[str]:
 # flags of single libraries beside HIPCC_FLAGS: name -> function that returns them
 EXTRA_FLAGS = {"engine_api": _python_flags}
 # libraries compiled once per value of a constant: name -> (constant, values built ahead)
-VARIANT_LIBRARIES = {"attention_mfma": ("HEAD_DIM", [16, 32, 48, 64, 80, 128, 256]),
+VARIANT_LIBRARIES = {"attention_mfma": ("HEAD_DIM", [16, 32, 48, 64, 80, 96, 128, 192, 256]),
                      "gemm": ("GATE_ACT", [1])}
 
 

@@ -208,10 +208,15 @@ def test_a_matrix_per_head(H, n_in, n_out, T, pad, dtype):
 
 @pytest.mark.parametrize("kernel", ["rows", "prefill", "decode-block", "decode-split"])
 @pytest.mark.parametrize("H,G,D,window,n_keys", [(6, 2, 32, 0, 150), (4, 4, 16, 37, 300),
-                                                 (3, 1, 64, 0, 700), (8, 2, 128, 72, 90)])
-def test_attention_kernels_work_on_the_scores(kernel, H, G, D, window, n_keys):
-    """Cap, bias by distance and sink in every attention kernel (bfloat16; the plain kernel also in
-    float32), one request of ``n_keys`` keys and a second short one, against the stand-in."""
+                                                 (3, 1, 64, 0, 700), (8, 2, 128, 72, 90),
+                                                 (5, 1, 96, 50, 200), (16, 1, 192, 0, 300),
+                                                 (4, 2, 48, 0, 130), (2, 1, 256, 64, 150)])
+@pytest.mark.parametrize("what", ["all", "sink"])
+def test_attention_kernels_work_on_the_scores(kernel, H, G, D, window, n_keys, what):
+    """Cap, bias by distance and sink (or the sink alone, which leaves the scores to the kernels'
+    plain path) in every attention kernel (bfloat16; the plain kernel also in float32), one
+    request of ``n_keys`` keys and a second short one, against the stand-in.  The bias table ends
+    40 keys back: most key tiles of the long request lie beyond it."""
     from kappai_amd.kernels import ops
     ps = 16
     lens = [n_keys, 21]
@@ -227,7 +232,11 @@ def test_attention_kernels_work_on_the_scores(kernel, H, G, D, window, n_keys):
             bt[s, b] = order[at]
             at += 1
     mods_host = ops.ScoreMods(2.5, torch.randn(H, 40, generator=g), torch.randn(H, generator=g) + 2)
-    mods = ops.ScoreMods(2.5, mods_host.distance_bias.to(DEV), mods_host.sink.to(DEV))
+    if what == "sink":
+        mods_host = ops.ScoreMods(0.0, None, mods_host.sink)
+    mods = ops.ScoreMods(mods_host.softcap,
+                         None if what == "sink" else mods_host.distance_bias.to(DEV),
+                         mods_host.sink.to(DEV))
     if kernel in ("decode-block", "decode-split"):
         segs = [(lens[0] - 1, 1), (lens[1] - 1, 1)]
     else:
@@ -252,7 +261,8 @@ def test_attention_kernels_work_on_the_scores(kernel, H, G, D, window, n_keys):
     # the sink alone changes the result (it is not dropped somewhere on the way)
     bare = E.paged_attention(q.float(), H, G, D, k_pool.float(), v_pool.float(), host["row_pos"],
                              host["row_seg"], bt, ps, 0.3, window=window,
-                             mods=ops.ScoreMods(2.5, mods_host.distance_bias, None)).double()
+                             mods=ops.ScoreMods(mods_host.softcap, mods_host.distance_bias,
+                                                None)).double()
     assert float((bare - want).abs().max()) > 0.05
 
 
