@@ -484,9 +484,9 @@ def test_delta_rule_overwrites_what_a_key_held():
 # ---------------------------------------------------------------------------------------------
 # whole models
 # ---------------------------------------------------------------------------------------------
-LENGTHS = {"U": [70, 45, 100, 37], "V": [66, 35, 90], "W": [50, 81, 36]}
+LENGTHS = {"U": [70, 45, 100, 37], "V": [66, 35, 90], "W": [50, 81, 36], "X": [130, 60, 90]}
 MIXED_LENGTHS = {"U": [70, 45, 100, 37, 83, 64, 29, 58], "V": [66, 35, 90, 41, 23, 77, 50, 62, 88],
-                 "W": [50, 81, 36, 67, 44, 72, 90, 33, 58]}
+                 "W": [50, 81, 36, 67, 44, 72, 90, 33, 58], "X": [130, 60, 90, 41, 75, 100, 33]}
 
 
 @pytest.fixture(scope="module")
@@ -525,7 +525,7 @@ def replay(model_dir, dtype, steps, index, max_tokens, out_dir, slots=4, graphs=
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["U", "V", "W"])
+@pytest.mark.parametrize("name", ["U", "V", "W", "X"])
 @pytest.mark.parametrize("family", ["whole", "prefill_then_decode", "changing_portions", "mixed"])
 def test_schedules(tmp_path, model_dirs, name, family, dtype):
     """Every logit of every request.  The mixed family runs in a pool smaller than its requests

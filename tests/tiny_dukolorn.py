@@ -76,7 +76,21 @@ TINY_W = config(150, 64, 1e-5, 0.125, [
 ])
 INIT_W = dict(seed=33, std=0.12, norm_jitter=0.0)
 
-TINY = {"U": (TINY_U, INIT_U), "V": (TINY_V, INIT_V), "W": (TINY_W, INIT_W)}
+# sizes in between: attention heads of 48, 80 and 96 once widened (two kv heads of 32 / 48, five
+# heads on a latent of 64 + 16, two on 64 + 32), four heads on one kv head, a window of 50, two
+# taps, three q/k heads for six value heads, a table whose linear half ends at 16
+TINY_X = config(500, 192, 1e-5, 0.7, [
+    parallel(6, 3, 32, 48, 0.17, 15.0, 10, 100.0, 0.25, 50, 4, 24, 40, 4.0, 6, 0.9, 0.6,
+             dense(256)),
+    latent(5, 32, 16, 40, 64, 0.14, 5000.0, 16, 50, dense(200)),
+    delta(6, 3, 48, 24, 2, 5, 5, None),
+    latent(2, 16, 32, 16, 64, 0.2, 20000.0, 32, None, dense(128)),
+    parallel(4, 1, 64, 64, 0.125, 50.0, 32, 64.0, 0.1, 40, 2, 64, 32, 16.0, 8, 1.0, 1.0, None),
+])
+INIT_X = dict(seed=34, std=0.08, norm_jitter=0.0)
+
+TINY = {"U": (TINY_U, INIT_U), "V": (TINY_V, INIT_V), "W": (TINY_W, INIT_W),
+        "X": (TINY_X, INIT_X)}
 
 
 def write_tiny(name: str, folder, **overrides):
