@@ -382,17 +382,24 @@ __global__ __launch_bounds__(LA_MAX_WAVES * WAVE) void matrix_state_scan_block_k
     const int nn = min(tb, last - t0 - tb);
     if (nn > 0) fetch(t0 + tb, nn);
     // two sets of registers take turns: one is read for the next token while the other is used
+    // (a read past the chunk's tokens stays inside the chunk's LDS or the next one's start, and
+    // what it brings is not used: the loop over pairs needs no tests inside)
     float q0[R], k0[R], a0[R], v0, b0, q1[R], k1[R], a1[R], v1, b1;
+    float* op = orow + (size_t)t0 * ostep;
     read(0, q0, k0, a0, v0, b0);
-    for (int tt = 0; tt < n; tt += 2) {
-      if (tt + 1 < n) read(tt + 1, q1, k1, a1, v1, b1);
+    int tt = 0;
+    for (; tt + 1 < n; tt += 2) {
+      read(tt + 1, q1, k1, a1, v1, b1);
       const float o0 = la_token<KS, R, DELTA>(S, q0, k0, a0, v0, b0);
-      if (writes) orow[(size_t)(t0 + tt) * ostep] = o0;
-      if (tt + 1 < n) {
-        if (tt + 2 < n) read(tt + 2, q0, k0, a0, v0, b0);
-        const float o1 = la_token<KS, R, DELTA>(S, q1, k1, a1, v1, b1);
-        if (writes) orow[(size_t)(t0 + tt + 1) * ostep] = o1;
-      }
+      if (writes) op[0] = o0;
+      read(min(tt + 2, tb - 1), q0, k0, a0, v0, b0);
+      const float o1 = la_token<KS, R, DELTA>(S, q1, k1, a1, v1, b1);
+      if (writes) op[ostep] = o1;
+      op += 2 * ostep;
+    }
+    if (tt < n) {
+      const float o0 = la_token<KS, R, DELTA>(S, q0, k0, a0, v0, b0);
+      if (writes) op[0] = o0;
     }
     __syncthreads();
     if (nn > 0) put(nn);
