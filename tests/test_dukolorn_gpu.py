@@ -285,7 +285,8 @@ def scored_dict(H, G, d, dv, **kw):
 
 
 @pytest.mark.parametrize("dtype,tol", [(F32, 2e-5), (BF16, 3e-2)])
-@pytest.mark.parametrize("H,G,d,dv", [(6, 2, 16, 24), (3, 3, 24, 16), (1, 1, 40, 8), (8, 1, 16, 16)])
+@pytest.mark.parametrize("H,G,d,dv", [(6, 2, 16, 24), (3, 3, 24, 16), (1, 1, 40, 8), (8, 1, 16, 16),
+                                      (18, 1, 16, 16), (40, 2, 8, 16)])
 def test_scored_attention_part(dtype, tol, H, G, d, dv):
     from kappai_amd.cache import CacheManager
     part = scored_part(dtype, H, G, d, dv)
@@ -371,7 +372,9 @@ def test_scored_attention_finds_a_far_key_and_weighs_bias_and_sink(dtype, tol):
 @pytest.mark.parametrize("H,d,rot,dv,r,dims,window", [(3, 16, 8, 24, 20, 8, 21),
                                                       (2, 8, 16, 8, 40, 12, None),
                                                       (4, 8, 8, 16, 24, 8, 1),
-                                                      (2, 24, 8, 8, 16, 8, 33)])
+                                                      (2, 24, 8, 8, 16, 8, 33),
+                                                      (20, 8, 8, 8, 16, 8, 21),
+                                                      (17, 16, 16, 8, 64, 16, None)])
 def test_latent_attention_part(dtype, tol, H, d, rot, dv, r, dims, window):
     from kappai_amd.cache import CacheManager
     from kappai_amd.parts import LatentAttention, RotaryEncoding
